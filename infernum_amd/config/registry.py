@@ -35,9 +35,10 @@ def resolve_architecture(model_type: str) -> Tuple[Any, Callable[..., Any]]:
 
 
 def config_from_dict(raw: Mapping[str, Any], where: str = "config.json") -> Any:
-    model_type = raw.get("model_type", DEFAULT_MODEL_TYPE)
+    # a file names its design in 'model_type' or, without one, in 'architecture'
+    model_type = raw.get("model_type", raw.get("architecture", DEFAULT_MODEL_TYPE))
     if not isinstance(model_type, str):
-        raise ConfigError(f"{where}: 'model_type' must be a string")
+        raise ConfigError(f"{where}: 'model_type' (or 'architecture') must be a string")
     config_cls, _ = resolve_architecture(model_type)
     return config_cls.from_dict(raw, where)
 

@@ -1,6 +1,6 @@
 // Causal attention of a ragged batch over paged keys and values, one wave per
 // (query token, query head), in fp32 throughout.  It serves the true 32-bit
-// path, and is the plain twin of the MFMA kernels.  Any head size up to 256,
+// path, and is the plain twin of the MFMA kernels.  Any head size up to 640,
 // any page size, any grouping of query heads over key/value heads, an optional
 // window.  Keys are summed in the order of their positions, 64 at a time, so the
 // result at a position does not depend on what else the batch holds.
@@ -10,7 +10,7 @@
 // sees keys max(0, pos - window + 1) .. pos  (window <= 0: all keys from 0).
 #include "common.h"
 
-#define AG_MAX_D 256
+#define AG_MAX_D 640
 
 template <typename T>
 __global__ __launch_bounds__(64) void attn_generic_kernel(const T* __restrict__ q, int q_row_stride,

@@ -41,10 +41,14 @@ CORE_SOURCES = [
     "gemm_skinny.hip",
     "gemm_mfma.hip",
     "attention_generic.hip",
+    "norm_branch.hip",
+    "activations.hip",
+    "latent.hip",
+    "moe.hip",
     "sampling.hip",
     "peaks.hip",
 ]
-HEADERS = ["common.h", "no_alloc.h", "op_call.h"]
+HEADERS = ["common.h", "no_alloc.h", "op_call.h", "tile_fma.h"]
 # The host library: plain C++ (cache bookkeeping, packing of a step), built with the C++ compiler.
 HOST_SOURCES = ["host_core.cpp", "step_program.cpp"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]

@@ -4,11 +4,11 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
-// out[n, :] = table[ids[n], :] widened to fp32 (the residual stream is fp32).
+// out[n, :] = table[ids[n], :] widened to fp32 (the residual stream is fp32), times `scale` in fp32.
 // An id outside [0, V) gives a row of NaN, never an access outside the table.
 template <typename T>
 __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                                    float* __restrict__ out, int H, int V) {
+                                                    float* __restrict__ out, int H, int V, float scale) {
   const int n = blockIdx.x;
   const int id = ids[n];
   float* o = out + (size_t)n * H;
@@ -19,8 +19,8 @@ __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table,
   const T* r = table + (size_t)id * H;
   // 16 bytes of the table at a time where rows allow it, all of a thread's loads issued before its first store
   constexpr int PER = 16 / (int)sizeof(T);              // values in 16 bytes
-  if (H % PER == 0 && (reinterpret_cast<uintptr_t>(table) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
-      H <= 256 * PER * 4) {
+  if (scale == 1.0f && H % PER == 0 && (reinterpret_cast<uintptr_t>(table) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && H <= 256 * PER * 4) {
     uint4 v[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -46,17 +46,17 @@ __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table,
     }
     return;
   }
-  for (int i = threadIdx.x; i < H; i += 256) o[i] = to_float(r[i]);
+  for (int i = threadIdx.x; i < H; i += 256) o[i] = to_float(r[i]) * scale;
 }
 
 extern "C" int ia_embed(const void* table, int table_dtype, const int* ids, float* out, int N, int H, int V,
-                        hipStream_t stream) {
-  if (N < 0 || H <= 0 || V <= 0) return IA_ERR_BAD_ARG;
+                        float scale, hipStream_t stream) {
+  if (N < 0 || H <= 0 || V <= 0 || !(scale == scale)) return IA_ERR_BAD_ARG;
   if (N == 0) return IA_OK;
   if (table_dtype == IA_F32)
-    embed_kernel<float><<<N, 256, 0, stream>>>((const float*)table, ids, out, H, V);
+    embed_kernel<float><<<N, 256, 0, stream>>>((const float*)table, ids, out, H, V, scale);
   else if (table_dtype == IA_BF16)
-    embed_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V);
+    embed_kernel<bf16_t><<<N, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V, scale);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

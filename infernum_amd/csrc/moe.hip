@@ -1,0 +1,218 @@
+// Routed experts: a token's feed-forward is the weighted sum of `top` small gated feed-forwards chosen among E.
+//   ia_router_topk   z = logits + bias (fp32); the `top` largest (the lowest index among equals) and the softmax
+//                    over those alone;
+//   ia_moe_sort      the (token, choice) pairs grouped by expert: offsets[E + 1], perm[P];
+//   ia_moe_gate_up   per expert, over its pairs' tokens: g = min(Wg x, limit), u = clamp(Wu x, -limit, limit),
+//                    y = g sigmoid(alpha g) (u + 1); the rows of Wg and Wu alternate in the expert's matrix;
+//   ia_moe_down      per expert: Wd y times the pair's routing weight, as fp32 into parts[choice, token, :], which
+//                    the kernel that takes the feed-forward's result next adds in the order of the choices.
+// Only the chosen experts' weights are read.  A pair's result is one chain of operations over its own token and
+// its expert's weights, whatever else the step holds and wherever the sort has put it.
+#include "common.h"
+#include "tile_fma.h"
+
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
+                                                          const void* __restrict__ bias, int bias_dtype,
+                                                          int* __restrict__ ids, float* __restrict__ weights, int N,
+                                                          int E, int top) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  const float* z = logits + (size_t)n * E;
+  float prev_v = INFINITY, first_v = 0.f, sum = 0.f;
+  int prev_i = -1;
+  for (int k = 0; k < top; ++k) {
+    float best_v = -INFINITY;
+    int best_i = -1;
+    for (int e = 0; e < E; ++e) {
+      const float v = z[e] + (bias ? load_as_float(bias, bias_dtype, e) : 0.f);
+      const bool after = (v < prev_v) || (v == prev_v && e > prev_i);       // not chosen yet
+      if (after && (best_i < 0 || v > best_v)) { best_v = v; best_i = e; }
+    }
+    if (best_i < 0) {          // values that compare with nothing (NaN): any expert not chosen yet, by index
+      best_i = prev_i + 1 < E ? prev_i + 1 : 0;
+      best_v = z[best_i];
+    }
+    if (k == 0) first_v = best_v;
+    const float w = expf(best_v - first_v);
+    ids[(size_t)n * top + k] = best_i;
+    weights[(size_t)n * top + k] = w;
+    sum += w;
+    prev_v = best_v;
+    prev_i = best_i;
+  }
+  const float inv = 1.0f / sum;
+  for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] *= inv;
+}
+
+extern "C" int ia_router_topk(const float* logits, const void* bias, int bias_dtype, int* ids, float* weights, int N,
+                              int E, int top, hipStream_t stream) {
+  if (N < 0 || E <= 0 || top <= 0 || top > E) return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  router_topk_kernel<<<(N + 255) / 256, 256, 0, stream>>>(logits, bias, bias_dtype, ids, weights, N, E, top);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+#define MOE_MAX_E 1024
+// One workgroup.  offsets[e] .. offsets[e + 1] - 1 are the places in perm of expert e's pairs; the order of an
+// expert's pairs is whatever the atomics give (no result depends on it).
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int* __restrict__ offsets,
+                                                        int* __restrict__ perm, int P, int E) {
+  __shared__ int cnt[MOE_MAX_E];
+  __shared__ int cur[MOE_MAX_E];
+  for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += 1024) {
+    const int e = ids[p];
+    if ((unsigned)e < (unsigned)E) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = at;
+      cur[e] = at;
+      at += cnt[e];
+    }
+    offsets[E] = at;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += 1024) {
+    const int e = ids[p];
+    if ((unsigned)e < (unsigned)E) perm[atomicAdd(&cur[e], 1)] = p;
+  }
+}
+
+extern "C" int ia_moe_sort(const int* ids, int* offsets, int* perm, int P, int E, hipStream_t stream) {
+  if (P < 0 || E <= 0) return IA_ERR_BAD_ARG;
+  if (E > MOE_MAX_E) return IA_ERR_UNSUPPORTED;
+  moe_sort_kernel<<<1, 1024, 0, stream>>>(ids, offsets, perm, P, E);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// Tile t of the launch (rows of 64 pairs, expert by expert): its expert and its first place in perm; false when
+// the launch has more tiles than the step needs.
+__device__ __forceinline__ bool moe_tile(const int* __restrict__ offsets, int E, int t, int& expert, int& first,
+                                         int& last) {
+  int seen = 0;
+  for (int e = 0; e < E; ++e) {
+    const int lo = offsets[e], hi = offsets[e + 1];
+    const int tiles = (hi - lo + TF_T - 1) / TF_T;
+    if (t < seen + tiles) {
+      expert = e;
+      first = lo + (t - seen) * TF_T;
+      last = hi;
+      return true;
+    }
+    seen += tiles;
+  }
+  return false;
+}
+
+// grid: (tiles of 2 * ff columns, ceil(P / 64) + E).  Wgu [E, 2 ff, W]: row 2 j the gate's row j, row 2 j + 1 up's.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ Wgu,
+                                                          T* __restrict__ y, const int* __restrict__ offsets,
+                                                          const int* __restrict__ perm, int E, int top, int W,
+                                                          int ff, float limit, float alpha) {
+  __shared__ TileFmaLds lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
+  const int n0 = blockIdx.x * TF_T;
+  const int lr = threadIdx.x >> 2;
+  const T* a_row = (first + lr < last) ? x + (size_t)(perm[first + lr] / top) * W : nullptr;
+  const T* w_row = (n0 + lr < 2 * ff) ? Wgu + ((size_t)e * 2 * ff + n0 + lr) * W : nullptr;
+  float acc[4][4];
+  tile_fma_64(a_row, w_row, W, acc, lds);
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = first + ty * 4 + i;
+    if (p >= last) continue;
+#pragma unroll
+    for (int j = 0; j < 4; j += 2) {
+      const int c = n0 + tx * 4 + j;
+      if (c + 1 >= 2 * ff) continue;
+      // both products are rounded as a stored tensor would be, then the activation in fp32
+      const float g = fminf(to_float(from_float<T>(acc[i][j])), limit);
+      const float u = fminf(fmaxf(to_float(from_float<T>(acc[i][j + 1])), -limit), limit);
+      y[(size_t)p * ff + (c >> 1)] = from_float<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+    }
+  }
+}
+
+extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int* offsets, const int* perm, int dtype,
+                              int P, int E, int top, int W, int ff, float limit, float alpha, hipStream_t stream) {
+  if (P < 0 || E <= 0 || top <= 0 || W <= 0 || ff <= 0) return IA_ERR_BAD_ARG;
+  if (P == 0) return IA_OK;
+  dim3 grid((2 * ff + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
+  if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
+  if (dtype == IA_F32)
+    moe_gate_up_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets, perm,
+                                                        E, top, W, ff, limit, alpha);
+  else if (dtype == IA_BF16)
+    moe_gate_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
+                                                         perm, E, top, W, ff, limit, alpha);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// grid: (tiles of W columns, ceil(P / 64) + E).  Wd [E, W, ff]; parts [top, N, W] fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ y, const T* __restrict__ Wd,
+                                                       float* __restrict__ parts, const float* __restrict__ weights,
+                                                       const int* __restrict__ offsets, const int* __restrict__ perm,
+                                                       int E, int top, int N, int W, int ff) {
+  __shared__ TileFmaLds lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
+  const int n0 = blockIdx.x * TF_T;
+  const int lr = threadIdx.x >> 2;
+  const T* a_row = (first + lr < last) ? y + (size_t)(first + lr) * ff : nullptr;
+  const T* w_row = (n0 + lr < W) ? Wd + ((size_t)e * W + n0 + lr) * ff : nullptr;
+  float acc[4][4];
+  tile_fma_64(a_row, w_row, ff, acc, lds);
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int p = first + ty * 4 + i;
+    if (p >= last) continue;
+    const int pair = perm[p];
+    const int token = pair / top, choice = pair - token * top;
+    const float wt = weights[pair];
+    float* o = parts + ((size_t)choice * N + token) * W;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = n0 + tx * 4 + j;
+      if (c < W) o[c] = to_float(from_float<T>(acc[i][j])) * wt;
+    }
+  }
+}
+
+extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const float* weights, const int* offsets,
+                           const int* perm, int dtype, int N, int E, int top, int W, int ff, hipStream_t stream) {
+  if (N < 0 || E <= 0 || top <= 0 || W <= 0 || ff <= 0) return IA_ERR_BAD_ARG;
+  if (N == 0) return IA_OK;
+  const int P = N * top;
+  dim3 grid((W + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
+  if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
+  if (dtype == IA_F32)
+    moe_down_kernel<float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets, perm,
+                                                     E, top, N, W, ff);
+  else if (dtype == IA_BF16)
+    moe_down_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
+                                                      perm, E, top, N, W, ff);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+#include "op_call.h"
+IA_OP(ia_router_topk)
+IA_OP(ia_moe_sort)
+IA_OP(ia_moe_gate_up)
+IA_OP(ia_moe_down)

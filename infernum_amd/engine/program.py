@@ -92,6 +92,12 @@ class Buffer:
             raise ProgramError(f"buffer {self.key!r} has no address before the program is finished")
         return self._program._arena.data_ptr() + self.offset
 
+    def at(self, nbytes: int) -> "BufferAt":
+        """The place ``nbytes`` into this buffer, as an argument of an operation (a head's part of a row, say)."""
+        if not 0 <= int(nbytes) <= self.nbytes:
+            raise ProgramError(f"buffer {self.key!r} holds {self.nbytes} bytes, a place {nbytes} bytes in was asked for")
+        return BufferAt(self, int(nbytes))
+
     def view(self, dtype: torch.dtype, *shape: int) -> torch.Tensor:
         """The first prod(shape) elements as a tensor (for operations written in Python)."""
         n = 1
@@ -101,6 +107,15 @@ class Buffer:
         if n * esz > self.nbytes:
             raise ProgramError(f"buffer {self.key!r} holds {self.nbytes} bytes, {n * esz} asked for")
         return self._program._arena[self.offset:self.offset + n * esz].view(dtype).view(*shape)
+
+
+class BufferAt:
+    """A place inside a :class:`Buffer` (``Buffer.at``)."""
+
+    __slots__ = ("buffer", "nbytes")
+
+    def __init__(self, buffer: Buffer, nbytes: int):
+        self.buffer, self.nbytes = buffer, nbytes
 
 
 def _term_not(t: Tuple) -> List[Tuple]:
@@ -479,6 +494,8 @@ class StepProgram:
             return [_ARG_PTR, a.index, 1, a.offset]
         if isinstance(a, Buffer):
             return [_ARG_CONST, 0, 1, a.ptr]
+        if isinstance(a, BufferAt):
+            return [_ARG_CONST, 0, 1, a.buffer.ptr + a.nbytes]
         if isinstance(a, torch.Tensor):
             if a.device != self._arena.device:
                 raise ProgramError(f"{name}: an operand is not on the program's device")

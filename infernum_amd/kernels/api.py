@@ -30,6 +30,7 @@ class KernelUnsupported(KernelError):
 
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+GENERIC_MAX_HEAD_DIM = 640         # the plain attention kernel's limit (AG_MAX_D)
 _libs: Dict[str, ctypes.CDLL] = {}
 
 _ERRORS = {10001: "bad argument", 10002: "size not supported by this kernel",
@@ -126,15 +127,16 @@ def _i32(t: torch.Tensor, n: int, what: str) -> None:
 
 
 # --------------------------------------------------------------------------- rows
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[n, :] = float(table[ids[n], :]); out is fp32 [N, H]."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[n, :] = float(table[ids[n], :]) * scale; out is fp32 [N, H]."""
     _dev(table, ids, out)
     V, H = table.shape
     N = ids.numel()
     _need(table.dtype in DTYPE_CODE, f"embed: table dtype {table.dtype}")
     _i32(ids, N, "embed ids")
     _need(out.dtype == torch.float32 and tuple(out.shape) == (N, H), f"embed: out must be fp32 [{N}, {H}]")
-    _ok(_core().ia_embed(_p(table), DTYPE_CODE[table.dtype], _p(ids), _p(out), N, H, V, _stream()), "embed")
+    _ok(_core().ia_embed(_p(table), DTYPE_CODE[table.dtype], _p(ids), _p(out), N, H, V, ctypes.c_float(scale),
+                         _stream()), "embed")
     return out
 
 
@@ -187,6 +189,132 @@ def add_rmsnorm(h: torch.Tensor, delta, weight: torch.Tensor, eps: float,
                                DTYPE_CODE[weight.dtype], _p(out), _p(rows), n_out, H, ctypes.c_float(eps),
                                _stream()), "add_rmsnorm")
     return out
+
+
+def norm_add(h: torch.Tensor, delta, weight: torch.Tensor, eps: float, x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h += delta * rsqrt(mean(delta^2) + eps) * weight (fp32, in place): the norm sits on the branch's output.
+
+    ``delta`` is a tensor of h's shape in the activations' dtype or a :class:`SplitSum`.  ``x`` (optional,
+    h's shape in the activations' dtype) receives the new h, rounded once: what the next sublayer reads."""
+    split = isinstance(delta, SplitSum)
+    d = delta.parts if split else delta
+    _dev(h, d, weight, x)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "norm_add: h must be fp32 [N, H]")
+    N, H = h.shape
+    splits, d_rows = 1, N
+    if split:
+        _need(d.shape[1] >= N and d.shape[2] == H, "norm_add: partial sums must be [S, >= N, H]")
+        splits, d_rows = d.shape[0], d.shape[1]
+    else:
+        _need(d is not None and d.dtype in DTYPE_CODE and tuple(d.shape) == (N, H), "norm_add: delta must have h's shape")
+    _need(weight.dtype in DTYPE_CODE and weight.numel() == H, f"norm_add: weight must hold {H} values")
+    act = x.dtype if x is not None else (torch.bfloat16 if d.dtype == torch.bfloat16 else torch.float32)
+    if x is not None:
+        _need(x.dtype in DTYPE_CODE and tuple(x.shape) == (N, H), "norm_add: x must have h's shape")
+        _need(split or x.dtype == d.dtype, "norm_add: x must have delta's dtype")
+    _ok(_core().ia_norm_add(_p(h), _p(d), DTYPE_CODE[d.dtype], splits, d_rows, _p(weight), DTYPE_CODE[weight.dtype],
+                            _p(x), DTYPE_CODE[act], N, H, ctypes.c_float(eps), _stream()), "norm_add")
+    return h
+
+
+ACTIVATIONS = {"gelu_tanh": 1}
+
+
+def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(x) element by element in fp32 (in place without ``out``).  Kinds: gelu_tanh."""
+    out = x if out is None else out
+    _dev(x, out)
+    _need(kind in ACTIVATIONS, f"activation: unknown kind {kind!r}; known: {sorted(ACTIVATIONS)}")
+    _need(x.dtype in DTYPE_CODE and out.dtype == x.dtype and out.numel() == x.numel(), "activation: out like x")
+    _ok(_core().ia_activation(_p(x), _p(out), DTYPE_CODE[x.dtype], ctypes.c_size_t(x.numel()), ACTIVATIONS[kind],
+                              _stream()), "activation")
+    return out
+
+
+def latent_prepare(proj: torch.Tensor, out: torch.Tensor, norm_weight: torch.Tensor, eps: float, H: int, dn: int,
+                   dr: int, rank: int) -> torch.Tensor:
+    """From rows [H heads of (dn plain | dr rotated) query values | rank latent values | dr key values | ...]
+    the rows [H heads of (dr | rank) | key (dr | rank) | value (dr | rank)] that the attention kernels take with
+    one key/value head: the rotated query parts at the heads' fronts (the rank places of the query heads are
+    left for :func:`gemm_heads`), key = (k_rot, c), value = (0, c), c = RMSNorm(latent) * norm_weight."""
+    _dev(proj, out, norm_weight)
+    N = proj.shape[0]
+    _need(proj.dim() == 2 and out.dim() == 2 and out.shape[0] == N and proj.dtype == out.dtype
+          and proj.dtype in DTYPE_CODE, "latent_prepare: two matrices of one dtype with the same rows")
+    _need(proj.shape[1] >= H * (dn + dr) + rank + dr and out.shape[1] >= (H + 2) * (dr + rank),
+          "latent_prepare: rows too short for their heads")
+    _need(norm_weight.dtype in DTYPE_CODE and norm_weight.numel() == rank, f"latent_prepare: {rank} norm weights")
+    _ok(_core().ia_latent_prepare(_p(proj), proj.shape[1], _p(out), out.shape[1], DTYPE_CODE[out.dtype],
+                                  _p(norm_weight), DTYPE_CODE[norm_weight.dtype], N, H, dn, dr, rank,
+                                  ctypes.c_float(eps), _stream()), "latent_prepare")
+    return out
+
+
+def gemm_heads(x: torch.Tensor, x_offset: int, x_head: int, w: torch.Tensor, out: torch.Tensor, out_offset: int,
+               out_head: int, gate: Optional[torch.Tensor] = None, gate_offset: int = 0) -> torch.Tensor:
+    """out[n, out_offset + h out_head + j] = sum_k x[n, x_offset + h x_head + k] w[h, j, k], for every head h of
+    w [H, J, K]; with ``gate`` times sigmoid(gate[n, gate_offset + h J + j]).  x, out and gate are matrices of one
+    dtype with the same rows; the offsets and head strides are in elements."""
+    _dev(x, w, out, gate)
+    _need(w.dim() == 3 and x.dim() == 2 and out.dim() == 2 and x.shape[0] == out.shape[0], "gemm_heads: shapes")
+    H, J, Kd = w.shape
+    N = x.shape[0]
+    _need(x.dtype == w.dtype == out.dtype and x.dtype in DTYPE_CODE, "gemm_heads: one dtype")
+    _need(x_offset >= 0 and x_offset + (H - 1) * x_head + Kd <= x.shape[1], "gemm_heads: x's rows are too short")
+    _need(out_offset >= 0 and out_offset + (H - 1) * out_head + J <= out.shape[1], "gemm_heads: out's rows are too short")
+    esz = x.element_size()
+    gp, g_row = None, 0
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.shape[0] == N and gate.dtype == x.dtype
+              and gate_offset >= 0 and gate_offset + H * J <= gate.shape[1], "gemm_heads: gate")
+        gp, g_row = ctypes.c_void_p(gate.data_ptr() + gate_offset * esz), gate.shape[1]
+    _ok(_core().ia_gemm_heads(ctypes.c_void_p(x.data_ptr() + x_offset * esz), x.shape[1], x_head, _p(w),
+                              ctypes.c_void_p(out.data_ptr() + out_offset * esz), out.shape[1], out_head,
+                              gp, g_row, DTYPE_CODE[x.dtype], N, H, J, Kd, _stream()), "gemm_heads")
+    return out
+
+
+def router_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """-> (ids int32 [N, top], weights fp32 [N, top]): the ``top`` largest of logits + bias per row (the lowest
+    index among equals) and the softmax over those alone."""
+    _dev(logits, bias)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "router_topk: fp32 logits [N, E]")
+    N, E = logits.shape
+    _need(0 < top <= E, f"router_topk: top must be 1 .. {E}")
+    _need(bias is None or (bias.dtype in DTYPE_CODE and bias.numel() == E), f"router_topk: {E} biases")
+    ids = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+    _ok(_core().ia_router_topk(_p(logits), _p(bias), DTYPE_CODE[bias.dtype] if bias is not None else 0, _p(ids),
+                               _p(weights), N, E, top, _stream()), "router_topk")
+    return ids, weights
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
+                w_down: torch.Tensor, limit: float, alpha: float) -> SplitSum:
+    """The chosen experts of every token: w_gate_up [E, 2 ff, W] with the gate's and up's rows alternating,
+    w_down [E, W, ff].  y = g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit).
+    Returns fp32 parts [top, N, W], each already times its routing weight."""
+    _dev(x, ids, weights, w_gate_up, w_down)
+    N, W = x.shape
+    E, two_ff, _ = w_gate_up.shape
+    ff = two_ff // 2
+    top = ids.shape[1]
+    _need(x.dtype in DTYPE_CODE and w_gate_up.dtype == x.dtype and w_down.dtype == x.dtype, "moe: one dtype")
+    _need(tuple(w_gate_up.shape) == (E, 2 * ff, W) and tuple(w_down.shape) == (E, W, ff), "moe: weights' shapes")
+    _need(ids.dtype == torch.int32 and tuple(ids.shape) == (N, top) and weights.dtype == torch.float32
+          and tuple(weights.shape) == (N, top), "moe: ids int32 and weights fp32 [N, top]")
+    P = N * top
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=x.device)
+    perm = torch.empty(max(P, 1), dtype=torch.int32, device=x.device)
+    y = torch.empty((max(P, 1), ff), dtype=x.dtype, device=x.device)
+    parts = torch.empty((top, N, W), dtype=torch.float32, device=x.device)
+    code = DTYPE_CODE[x.dtype]
+    _ok(_core().ia_moe_sort(_p(ids), _p(offsets), _p(perm), P, E, _stream()), "moe_sort")
+    _ok(_core().ia_moe_gate_up(_p(x), _p(w_gate_up), _p(y), _p(offsets), _p(perm), code, P, E, top, W, ff,
+                               ctypes.c_float(limit), ctypes.c_float(alpha), _stream()), "moe_gate_up")
+    _ok(_core().ia_moe_down(_p(y), _p(w_down), _p(parts), _p(weights), _p(offsets), _p(perm), code, N, E, top, W, ff,
+                            _stream()), "moe_down")
+    return SplitSum(parts)
 
 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
@@ -552,7 +680,7 @@ def attention_generic(qkv: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.T
     N = out.shape[0]
     _i32(token_seq, N, "attention token_seq")
     _i32(positions, N, "attention positions")
-    _need(0 < d <= 256, "attention: head size must be at most 256")
+    _need(0 < d <= GENERIC_MAX_HEAD_DIM, f"attention: head size must be at most {GENERIC_MAX_HEAD_DIM}")
     _ok(_core().ia_attention_generic(_p(qkv), qkv.shape[1], _p(k_pages), _p(v_pages), _p(out), nh * d,
                                      DTYPE_CODE[out.dtype], _p(token_seq), _p(positions), _p(block_tables),
                                      block_tables.shape[1], N, nh, nkv, d, k_pages.shape[2], k_pages.shape[0],

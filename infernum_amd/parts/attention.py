@@ -54,8 +54,8 @@ class Attention(Mixer):
         super().__init__(rt)
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
-        if head_dim > 256:
-            raise ValueError(f"head size {head_dim} is above 256, the largest the attention kernels take")
+        if head_dim > K.GENERIC_MAX_HEAD_DIM:
+            raise ValueError(f"head size {head_dim} is above {K.GENERIC_MAX_HEAD_DIM}, the largest the attention kernels take")
         self.hidden_size, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.window = int(window) if window else 0
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
@@ -127,69 +127,92 @@ class Attention(Mixer):
         nh, nkv, d = self.nh, self.nkv, self.d
         if cache.k_pages is None:
             raise K.KernelError("attention needs pages of the cache")
-        g = cache.group
-        if (self.use_mfma and self.rotate_in_attention and 0 < ctx.num_decode == x.shape[0] and self.qk_transform is None
-                and x.shape[0] <= ROTATE_IN_ATTENTION_UP_TO and cache.k_pages.shape[2] % 4 == 0):
-            # every request brings one token: rotation, the write to the pages and attention are one launch
-            w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
+        # keys and values of another run of a layer: only queries are made here
+        w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
+        if self.qk_transform is not None:
+            qkv = self.qk_transform.forward(linear(x, w, kernels=self.rt.kernels), nh, nkv if cache.writable else 0, d, ctx)
+        else:
             qkv = linear(x, w, keep_split=True, kernels=self.rt.kernels)
-            out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+        out = self.rotate_attend(qkv, ctx, cache)
+        return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
+
+    def rotate_attend(self, qkv, ctx: StepContext, cache: CacheView, transformed: Optional[bool] = None) -> torch.Tensor:
+        """From the rows [nh query heads | nkv key heads | nkv value heads] (a tensor or a SplitSum; queries only
+        when the pages are another run's): rotation, the write of keys and values to their pages, attention.
+        Returns [N, nh d].  Mixers that come by such rows another way than by one projection use it too."""
+        nh, nkv, d = self.nh, self.nkv, self.d
+        g = cache.group
+        n = qkv.shape[0]
+        dtype = self.rt.dtype
+        transformed = (self.qk_transform is not None) if transformed is None else transformed
+        if (self.use_mfma and self.rotate_in_attention and 0 < ctx.num_decode == n and not transformed
+                and n <= ROTATE_IN_ATTENTION_UP_TO and cache.k_pages.shape[2] % 4 == 0):
+            # every request brings one token: rotation, the write to the pages and attention are one launch
+            out = torch.empty((n, nh * d), dtype=dtype, device=cache.k_pages.device)
             K.attention_decode_rotating(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                                         ctx.slots[g] if cache.writable else None, cache.k_pages, cache.v_pages, out,
                                         ctx.block_tables[g], nh, nkv, d, self.scale, self.window, ctx.max_total_len)
-            return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
+            return out
         q_out = None
-        if self.qk_transform is not None:
-            w = self.w_qkv if cache.writable else self.w_qkv[: nh * d]
-            qkv = self.qk_transform.forward(linear(x, w, kernels=self.rt.kernels), nh, nkv if cache.writable else 0, d, ctx)
-            if cache.writable:
-                q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
-                                     ctx.slots[g], cache.k_pages, cache.v_pages)
-            else:
-                q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim)
-        elif cache.writable:
-            qkv = linear(x, self.w_qkv, keep_split=True, kernels=self.rt.kernels)
-            if isinstance(qkv, K.SplitSum):
-                q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+        if isinstance(qkv, K.SplitSum):
+            q_out = torch.empty((n, nh * d), dtype=dtype, device=cache.k_pages.device)
+        if cache.writable:
             q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
                                  ctx.slots[g], cache.k_pages, cache.v_pages, q_out=q_out)
         else:
-            # keys and values of another run of a layer: only queries are made here
-            qkv = linear(x, self.w_qkv[: nh * d], keep_split=True, kernels=self.rt.kernels)
-            if isinstance(qkv, K.SplitSum):
-                q_out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
             q = K.rope_kv_append(qkv, ctx.positions, self.position.inv_freq, nh, nkv, d, self.position.rotary_dim,
                                  q_out=q_out)
-        out = torch.empty((x.shape[0], nh * d), dtype=x.dtype, device=x.device)
+        out = torch.empty((n, nh * d), dtype=dtype, device=cache.k_pages.device)
         self.attend(q, out, ctx, cache)
-        return linear(out, self.w_o, keep_split=True, kernels=self.rt.kernels)
+        return out
 
     def native(self, program, view: CacheView) -> None:
-        """The launches of ``forward`` and ``attend``, each with the steps it is for: steps of up to
-        ROTATE_IN_ATTENTION_UP_TO single tokens take the kernel that rotates, writes the pages and attends in one
-        launch; all others the rotary kernel, then the kernel for single tokens on the first rows and the one for
-        portions of prompts on the rest (or the plain kernel on all rows)."""
-        if type(self).forward is not Attention.forward or type(self).attend is not Attention.attend:
+        """The launches of ``forward``: the projection, :meth:`emit_rotate_attend`, the output projection."""
+        if (type(self).forward is not Attention.forward or type(self).attend is not Attention.attend
+                or type(self).rotate_attend is not Attention.rotate_attend):
             return super().native(program, view)              # a subclass that computes something else
-        from ..engine.program import NEVER, STREAM, Guard
         if view is None or view.k_pages is None or view.v_pages is None:
             raise K.KernelError("attention needs pages of the cache")
+        nh, d, rt = self.nh, self.d, self.rt
+        w = self.w_qkv if view.writable else self.w_qkv[: nh * d]     # another run's keys and values: only queries are made
+        row = int(w.shape[0])
+        program.keep(w)
+        qkv = emit_linear(program, program.x, program.N, w, rt.dtype, None, self.qk_transform is None, "attention.qkv",
+                          "attention.qkv")
+        if self.qk_transform is not None:
+            where, transform, kv_heads = qkv.tensor(), self.qk_transform, (self.nkv if view.writable else 0)
+
+            def between_projection_and_rotation(ctx: StepContext) -> None:
+                t = where.view(rt.dtype, ctx.num_tokens, row)
+                y = transform.forward(t, nh, kv_heads, d, ctx)
+                if y.data_ptr() != t.data_ptr():
+                    t.copy_(y)
+            program.python(between_projection_and_rotation, type(transform).__name__)
+        out = self.emit_rotate_attend(program, view, qkv, row, self.qk_transform is not None)
+        program.pending = emit_linear(program, out, program.N, self.w_o, rt.dtype, None, True, "attention.mix", "attention.o")
+
+    def emit_rotate_attend(self, program, view: CacheView, qkv, row: int, transformed: bool = False):
+        """The launches of :meth:`rotate_attend` and :meth:`attend` for the rows ``qkv`` (a Value of ``row`` columns),
+        each with the steps it is for: steps of up to ROTATE_IN_ATTENTION_UP_TO single tokens take the kernel that
+        rotates, writes the pages and attends in one launch; all others the rotary kernel, then the kernel for
+        single tokens on the first rows and the one for portions of prompts on the rest (or the plain kernel on all
+        rows).  Returns the buffer [N, nh d] of the attended rows."""
+        from ..engine.program import NEVER, STREAM, Guard
         nh, nkv, d, window, rt = self.nh, self.nkv, self.d, self.window, self.rt
         k, v, g, writable = view.k_pages, view.v_pages, view.group, view.writable
         ps, num_pages = int(k.shape[2]), int(k.shape[0])
         inv_freq = self.position.inv_freq
         rot = self.position.rotary_dim if inv_freq is not None else 0
         f64 = int(inv_freq is not None and inv_freq.dtype == torch.float64)
-        w = self.w_qkv if writable else self.w_qkv[: nh * d]     # another run's keys and values: only queries are made
-        row, T, N = int(w.shape[0]), program.T, program.N
+        T, N = program.T, program.N
         act, scale = program.act_code, float(self.scale)
         mfma = self.use_mfma and ps % 4 == 0
-        program.keep(k, v, inv_freq, w)
+        program.keep(k, v, inv_freq)
         bt, bt_cols = program.block_table(g), program.bt_cols(g)
         slots = program.slots(g) if writable else None
         out = program.buffer("attention.out", T * nh * d * program.act_bytes)
         fused = NEVER
-        if mfma and self.rotate_in_attention and self.qk_transform is None:
+        if mfma and self.rotate_in_attention and not transformed:
             fused = Guard.between(program.NPT, 0, 0) & Guard.between(N, 1, ROTATE_IN_ATTENTION_UP_TO)
         separate = ~fused
         if mfma:
@@ -218,17 +241,6 @@ class Attention(Mixer):
             splits = program.scalar(("attention: parts of the keys", nh, nkv, g, ps), parts_of_the_keys)
             shape = program.scalar(("attention: launch shape", nh, nkv, d, window), launch_shape)
             tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
-        qkv = emit_linear(program, program.x, N, w, rt.dtype, None, self.qk_transform is None, "attention.qkv",
-                          "attention.qkv")
-        if self.qk_transform is not None:
-            where, transform, kv_heads = qkv.tensor(), self.qk_transform, (nkv if writable else 0)
-
-            def between_projection_and_rotation(ctx: StepContext) -> None:
-                t = where.view(rt.dtype, ctx.num_tokens, row)
-                y = transform.forward(t, nh, kv_heads, d, ctx)
-                if y.data_ptr() != t.data_ptr():
-                    t.copy_(y)
-            program.python(between_projection_and_rotation, type(transform).__name__)
         for alt in qkv.alts:
             src, code, parts = alt.where, (K.DTYPE_CODE[torch.float32] if alt.splits else act), (alt.splits or 1)
             if mfma:
@@ -256,7 +268,7 @@ class Attention(Mixer):
                        [q, q_stride, k, v, out, nh * d, program.seq_starts, program.seq_ctx, bt, bt_cols, tiles, num_tiles,
                         nh, nkv, ps, num_pages, scale, window, shape, STREAM],
                        alt.when & separate & Guard.between(program.NP, 1))
-        program.pending = emit_linear(program, out, N, self.w_o, rt.dtype, None, True, "attention.mix", "attention.o")
+        return out
 
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d

@@ -5,6 +5,13 @@
 delta into the next norm, which adds and normalises in one pass over the row
 (the reference's add_rmsnorm fusion, infernum/src/graph/optimizer.rs:105-174,
 there limited to adds with one consumer).
+
+``branchnorm``: h' = h + norm1(mixer(h)); h'' = h' + norm2(feed_forward(h')).  The
+sublayers read the residual stream itself (rounded once to the compute dtype for
+their matrix products) and the norm sits on each branch's output; the
+feed-forward (with its norm) may be absent.  One kernel normalises the branch,
+adds it into the fp32 stream and leaves the rounded stream for the next
+sublayer (``RMSNorm.add_normed``).
 """
 from __future__ import annotations
 
@@ -33,4 +40,51 @@ class PreNormBlock(Block):
         self.feed_forward.native(program, None)
 
 
+class BranchNormBlock(Block):
+    graph_safe = True
+
+    def _stream_rows(self, h: torch.Tensor, pending, ctx: StepContext) -> torch.Tensor:
+        """The residual stream in the compute dtype: what the layer before left, or a cast of h."""
+        from ..kernels import api as K
+        if pending is not None:                         # a layer of another arrangement left its delta unadded
+            K.residual_add(h, pending.joined(self.rt.dtype) if isinstance(pending, K.SplitSum) else pending)
+            ctx.extras.pop("branchnorm.x", None)
+        kept = ctx.extras.get("branchnorm.x")
+        if kept is not None and kept[0] is h:
+            return kept[1]
+        return K.cast(h, self.rt.dtype)
+
+    def forward(self, h: torch.Tensor, pending, ctx: StepContext, cache: CacheView):
+        x = self._stream_rows(h, pending, ctx)
+        a = self.mixer.forward(x, ctx, cache)
+        x = torch.empty_like(x)
+        self.mixer_norm.add_normed(h, a, x)
+        if self.feed_forward is not None:
+            f = self.feed_forward.forward(x, ctx)
+            x = torch.empty_like(x)
+            self.feed_forward_norm.add_normed(h, f, x)
+        ctx.extras["branchnorm.x"] = (h, x)             # the next layer of this arrangement reads it
+        return None
+
+    def native(self, program, view: CacheView) -> None:
+        if type(self).forward is not BranchNormBlock.forward:
+            return super().native(program, view)
+        from ..engine.program import STREAM
+        from ..kernels import api as K
+        H = program.hidden_size
+        if program.pending is not None or getattr(program, "x_holds_stream", None) is not program.h:
+            if program.pending is not None:
+                raise K.KernelError("branchnorm after an arrangement that leaves its delta unadded is not written "
+                                    "as launches")
+            program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], program.x, program.act_code,
+                                           program.N * H, STREAM])
+        self.mixer.native(program, view)
+        self.mixer_norm.native_branch(program)
+        if self.feed_forward is not None:
+            self.feed_forward.native(program, None)
+            self.feed_forward_norm.native_branch(program)
+        program.x_holds_stream = program.h              # program.x is the stream, rounded, until a norm writes it
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "branchnorm", BranchNormBlock)

@@ -1,6 +1,6 @@
 """Token embedding and output head.
 
-h[t] = E[ids[t]] without scaling (infernum-llama/src/graph_builder.rs:442);
+h[t] = E[ids[t]] (infernum-llama/src/graph_builder.rs:442; times ``scale`` where a model has one);
 logits = f W^T for the wanted rows only, in fp32 straight from the fp32
 accumulators (:533-536).  When the file has no head matrix, the embedding
 matrix stands in: the reference decides that by the file's contents, not by
@@ -20,28 +20,32 @@ from .linear import emit_linear, linear
 
 class TokenEmbedding(Embedding):
     graph_safe = True
-    def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02):
+    def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0,
+                 name: str = "weight"):
+        """``scale`` multiplies the looked-up row in fp32 (the table itself stays as stored: a head tied to it
+        reads it unscaled); ``name`` is the table's local tensor name."""
         super().__init__(rt)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.init_std = init_std
+        self.scale, self.name = float(scale), str(name)
         self.table: Optional[torch.Tensor] = None
 
     def weights(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
+        return {self.name: WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std))}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.table = tensors["weight"].contiguous()
+        self.table = tensors[self.name].contiguous()
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
-        return K.embed(self.table, ctx.token_ids, h)
+        return K.embed(self.table, ctx.token_ids, h, self.scale)
 
     def native(self, program, view=None) -> None:
         if type(self).forward is not TokenEmbedding.forward:
             return super().native(program, view)
         from ..engine.program import STREAM
         program.op("core", "ia_embed", [self.table, K.DTYPE_CODE[self.table.dtype], program.token_ids, program.h,
-                                        program.N, self.hidden_size, self.vocab_size, STREAM])
+                                        program.N, self.hidden_size, self.vocab_size, float(self.scale), STREAM])
         program.pending = None
 
 

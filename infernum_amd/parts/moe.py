@@ -1,0 +1,102 @@
+"""Routed experts: every token's feed-forward is the weighted sum of ``top`` of E small gated feed-forwards.
+
+  z = R x + b            router logits in fp32 (x as the matrix products read it), bias optional
+  chosen = the ``top`` largest z (lowest index among equals);  weight = softmax over the chosen z alone
+  expert e:  g = min(G_e x, limit),  u = clamp(U_e x, -limit, limit),  y = g sigmoid(alpha g) (u + 1),  D_e y
+  out = sum over the chosen, in the order of the choices, of weight * expert(x)
+
+``limit`` and ``alpha`` are parameters (alpha = 1.702 is the sigmoid form of GELU).  The experts' matrices are
+kept stacked, [E, 2 ff, W] with the rows of G_e and U_e alternating (so that a gate value and its up value
+end in one thread of the product's tile) and [E, W, ff].  The tokens are grouped by expert on the device, and
+only the chosen experts' weights are read.  The result is left as fp32 parts [top, N, W], one per choice, each
+already times its weight, which the next norm adds in the order of the choices: an expert's output is never
+rounded to the compute dtype.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import api as K
+from .base import FeedForward, Runtime, StepContext, WeightSpec, register_part
+from .linear import emit_linear, linear
+
+
+class RoutedExperts(FeedForward):
+    graph_safe = True
+
+    def __init__(self, rt: Runtime, hidden_size: int, intermediate_size: int, num_experts: int, top: int,
+                 limit: float, alpha: float = 1.702, router_bias: bool = True, router_name: str = "router",
+                 expert_prefix: str = "e", init_std: float = 0.02):
+        super().__init__(rt)
+        self.hidden_size, self.ff = int(hidden_size), int(intermediate_size)
+        self.num_experts, self.top = int(num_experts), int(top)
+        if not 0 < self.top <= self.num_experts:
+            raise ValueError(f"a token takes {top} of {num_experts} experts")
+        self.limit, self.alpha = float(limit), float(alpha)
+        if not self.limit > 0:
+            raise ValueError("the experts' limit must be positive")
+        self.router_bias, self.router_name, self.expert_prefix = bool(router_bias), router_name, expert_prefix
+        self.init_std = init_std
+        self.w_router: Optional[torch.Tensor] = None
+        self.b_router: Optional[torch.Tensor] = None
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def weights(self) -> Dict[str, WeightSpec]:
+        H, I, E = self.hidden_size, self.ff, self.num_experts
+        init = ("normal", self.init_std)
+        out = {self.router_name: WeightSpec((E, H), init)}
+        if self.router_bias:
+            out[self.router_name + ".b"] = WeightSpec((E,), ("normal", 0.5), follows_compute_dtype=False)
+        for e in range(E):
+            p = f"{self.expert_prefix}{e}."
+            out[p + "gate"] = WeightSpec((I, H), init)
+            out[p + "up"] = WeightSpec((I, H), init)
+            out[p + "down"] = WeightSpec((H, I), init)
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        H, I, E = self.hidden_size, self.ff, self.num_experts
+        self.w_router = tensors[self.router_name].contiguous()
+        self.b_router = tensors[self.router_name + ".b"].contiguous() if self.router_bias else None
+        dev, dt = self.w_router.device, self.w_router.dtype
+        self.w_gate_up = torch.empty((E, 2 * I, H), dtype=dt, device=dev)
+        self.w_down = torch.empty((E, H, I), dtype=dt, device=dev)
+        for e in range(E):
+            p = f"{self.expert_prefix}{e}."
+            self.w_gate_up[e, 0::2] = tensors[p + "gate"]
+            self.w_gate_up[e, 1::2] = tensors[p + "up"]
+            self.w_down[e] = tensors[p + "down"]
+
+    def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):
+        z = linear(x, self.w_router, out_dtype=torch.float32, kernels=self.rt.kernels)
+        ids, weights = K.router_topk(z, self.b_router, self.top)
+        return K.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, self.limit, self.alpha)
+
+    def native(self, program, view=None) -> None:
+        if type(self).forward is not RoutedExperts.forward:
+            return super().native(program, view)
+        from ..engine.program import ALWAYS, STREAM, Alt, Value
+        H, I, E, top, T, N = self.hidden_size, self.ff, self.num_experts, self.top, program.T, program.N
+        program.keep(self.w_router, self.b_router, self.w_gate_up, self.w_down)
+        z = emit_linear(program, program.x, N, self.w_router, torch.float32, None, False, "moe.logits", "moe.router")
+        ids = program.buffer("moe.ids", T * top * 4)
+        wts = program.buffer("moe.weights", T * top * 4)
+        offsets = program.buffer("moe.offsets", (E + 1) * 4)
+        perm = program.buffer("moe.perm", T * top * 4)
+        y = program.buffer("moe.y", T * top * I * program.act_bytes)
+        parts = program.buffer("moe.parts", top * T * H * 4)
+        b = self.b_router
+        program.op("core", "ia_router_topk", [z.tensor(), b, K.DTYPE_CODE[b.dtype] if b is not None else 0, ids, wts,
+                                              N, E, top, STREAM])
+        program.op("core", "ia_moe_sort", [ids, offsets, perm, N * top, E, STREAM])
+        program.op("core", "ia_moe_gate_up", [program.x, self.w_gate_up, y, offsets, perm, program.act_code, N * top,
+                                              E, top, H, I, self.limit, self.alpha, STREAM])
+        program.op("core", "ia_moe_down", [y, self.w_down, parts, wts, offsets, perm, program.act_code, N, E, top, H,
+                                           I, STREAM])
+        program.pending = Value(H, [Alt(ALWAYS, parts, top, torch.float32)])
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)
