@@ -114,10 +114,14 @@ def expert(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Te
 
 
 def routed_experts(h: torch.Tensor, w: Dict[str, torch.Tensor], mlp: dict,
-                   round_to: Optional[torch.dtype] = None) -> torch.Tensor:
+                   round_to: Optional[torch.dtype] = None, margins: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+    """``margins`` collects, per token, by how much the last chosen logit beats the first that is not chosen."""
     hr = _r(h, round_to)
     E, top, limit = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["limit"]
     idx, wt = route(hr, w["router"], w["router.b"], top)
+    if margins is not None and top < E:
+        z = (hr @ w["router"].t() + w["router.b"]).sort(dim=-1, descending=True).values
+        margins.append(z[:, top - 1] - z[:, top])
     out = torch.zeros_like(h)
     for e in range(E):
         rows, slot = (idx == e).nonzero(as_tuple=True)
@@ -133,8 +137,10 @@ def _local(weights: Dict[str, torch.Tensor], prefix: str, dtype) -> Dict[str, to
 
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int], dtype=torch.float64,
-            round_to: Optional[torch.dtype] = None, layers_out: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one sequence; ``layers_out`` collects the residual stream after every layer."""
+            round_to: Optional[torch.dtype] = None, layers_out: Optional[List[torch.Tensor]] = None,
+            margins: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+    """Logits [T, vocab] of one sequence; ``layers_out`` collects the residual stream after every layer,
+    ``margins`` the routers' margins (see ``routed_experts``) of every routed layer."""
     eps = cfg["norm"]["eps"]
     E = weights["embed"].to(dtype)
     x = E[torch.as_tensor(list(tokens), dtype=torch.long)] * cfg["embedding"]["scale"]
@@ -147,7 +153,7 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int], 
         mlp = layer.get("mlp")
         if mlp is not None:
             wl = _local(weights, p + "mlp.", dtype)
-            f = dense_ff(x, wl, round_to) if mlp["kind"] == "dense" else routed_experts(x, wl, mlp, round_to)
+            f = dense_ff(x, wl, round_to) if mlp["kind"] == "dense" else routed_experts(x, wl, mlp, round_to, margins)
             x = x + offset_norm(f, weights[p + "norm2"].to(dtype), eps)
         if layers_out is not None:
             layers_out.append(x.clone())
