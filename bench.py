@@ -435,6 +435,105 @@ def decode_kernels_alone(a) -> int:
     return 0
 
 
+# ---- the Nesilorn design beside the Llama decoder at equal sizes ------------------------------------------------
+# Layer sizes that resemble a real model's: the latent head (rotated part + latent) is 256 wide, the largest the
+# matrix-core attention kernels take; dense and routed feed-forwards alternate; the Llama twin has the same width,
+# layers, vocabulary and heads, and feed-forward matrices of as many parameters as a token uses here.
+NESILORN_SIZES = {
+    "2k": dict(width=2048, heads=16, dim=64, rot_dim=32, vdim=64, kv_rank=224, window=1024, dense_ff=8192, experts=32,
+               top=4, expert_ff=1408, layers=8, vocab=32000, llama_ff=5504, llama_kv_heads=4),
+    "4k": dict(width=4096, heads=32, dim=64, rot_dim=32, vdim=64, kv_rank=224, window=2048, dense_ff=14336, experts=32,
+               top=4, expert_ff=2432, layers=8, vocab=32000, llama_ff=9600, llama_kv_heads=8),
+}
+
+
+def nesilorn_configs(size: dict):
+    from infernum_amd.config import LlamaConfig, NesilornConfig
+    mixer = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot_dim"], "vdim": size["vdim"],
+             "kv_rank": size["kv_rank"], "scale": (size["dim"] + size["rot_dim"]) ** -0.5,
+             "rot": {"base": 10000.0, "dims": size["rot_dim"]}, "mask": {"size": size["window"]}}
+    dense = {"kind": "dense", "ff": size["dense_ff"]}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"], "limit": 7.0},
+           "router": {"experts": size["experts"], "top": size["top"]}}
+    nes = NesilornConfig.from_dict({
+        "architecture": "Nesilorn", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+        "norm": {"eps": 1e-6},
+        "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe}
+                   for i in range(size["layers"])]})
+    llama = LlamaConfig.from_dict(dict(
+        model_type="mistral", num_hidden_layers=size["layers"], hidden_size=size["width"],
+        num_attention_heads=size["heads"], num_key_value_heads=size["llama_kv_heads"],
+        intermediate_size=size["llama_ff"], vocab_size=size["vocab"], rope_theta=10000.0, rms_norm_eps=1e-6,
+        tie_word_embeddings=True, max_position_embeddings=8192, sliding_window=size["window"], use_sliding_window=True))
+    return nes, llama
+
+
+def nesilorn_active_params(size: dict) -> int:
+    """Weights that a token multiplies with in the Nesilorn model of these sizes (the head included)."""
+    W, H = size["width"], size["heads"]
+    mixer = (W * (H * (size["dim"] + size["rot_dim"]) + size["kv_rank"] + size["rot_dim"] + H * size["vdim"])
+             + H * size["kv_rank"] * (size["dim"] + size["vdim"]) + W * H * size["vdim"])
+    dense = 2 * W * size["dense_ff"]
+    routed = W * size["experts"] + size["top"] * 3 * W * size["expert_ff"]
+    n = size["layers"]
+    return n * mixer + (n - n // 2) * dense + (n // 2) * routed + size["vocab"] * W
+
+
+def nesilorn_bench(a) -> int:
+    """Prefill of 2,048 tokens and decode steps at batch 8 and 64 of the Nesilorn design and of the Llama decoder
+    at equal sizes, random weights, through the same engine and generation loop; one JSON line of its own."""
+    import torch
+    from infernum_amd import CacheConfig, Engine
+    from infernum_amd.engine import StepEntry
+    out = {"metric": "Nesilorn beside Llama at equal sizes", "dtype": "bf16", "data": "synthetic", "sizes": {}}
+    batches = [int(b) for b in a.nesilorn_batches.split(",") if b]
+    for name in a.nesilorn.split(","):
+        size = NESILORN_SIZES[name]
+        rec = {"config": {k: v for k, v in size.items()}}
+        for label, cfg in zip(("nesilorn", "llama"), nesilorn_configs(size)):
+            max_batch = max(batches)
+            tokens = max(max_batch * (PROMPT_LEN + a.steps + a.warmup + prefill_steps(max_batch, PROMPT_LEN) + 2 * PAGE_SIZE),
+                         PREFILL_TOKENS + PAGE_SIZE)
+            engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens_per_step=8192,
+                                        cache_config=CacheConfig(page_size=PAGE_SIZE, num_state_slots=max_batch + 1,
+                                                                 num_pages=tokens // PAGE_SIZE + max_batch))
+            sync()
+            r = {}
+            g = torch.Generator().manual_seed(7)
+            prompt = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=g).tolist()
+            best = None
+            for i in range(4):
+                sync()
+                t0 = time.perf_counter()
+                engine.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
+                sync()
+                t = time.perf_counter() - t0
+                engine.end(f"p{i}")
+                if i > 0:
+                    best = t if best is None else min(best, t)
+            r["prefill_2048_tok_per_s"] = round(PREFILL_TOKENS / best, 1)
+            r["prefill_2048_ms"] = round(best * 1e3, 3)
+            for b in batches:
+                steps = max(16, min(a.steps, 64))
+                dt, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)), PROMPT_LEN)
+                r[f"decode_b{b}_tok_per_s"] = round(b * steps / dt, 1)
+                r[f"decode_b{b}_ms_per_step"] = round(dt / steps * 1e3, 3)
+            if label == "nesilorn":
+                active = nesilorn_active_params(size)
+            else:
+                per_layers, head = matmul_params(cfg)
+                active = per_layers + head
+            r["active_params_m"] = round(active / 1e6, 1)
+            r["prefill_gemm_tflops"] = round(2.0 * active * PREFILL_TOKENS / best / 1e12, 1)
+            rec[label] = r
+            print(f"[bench] {name} {label}: {r}", file=sys.stderr, flush=True)
+            del engine
+            torch.cuda.empty_cache()
+        out["sizes"][name] = rec
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -468,11 +567,17 @@ def main() -> int:
                     help="tokens of a step, decoded ones and portions together (default: the larger of chunk and batch: a step of\n"
                          "2,048 rows fills the library's tiles of 256, one of 2,100 pays for 2,304)")
     ap.add_argument("--serve-blocks", type=int, default=16384)
+    ap.add_argument("--nesilorn", default="", metavar="SIZES",
+                    help="the Nesilorn design (latent attention, routed experts) beside the Llama decoder at equal sizes "
+                         "instead: prefill and decode of each (a JSON line of its own); sizes: 2k, 4k or both with a comma")
+    ap.add_argument("--nesilorn-batches", default="8,64", help="decode batches of --nesilorn")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
         return 2
 
+    if a.nesilorn:
+        return nesilorn_bench(a)
     if a.decode_kernels:
         return decode_kernels_alone(a)
     if a.serve:

@@ -66,37 +66,34 @@ extern "C" int ia_latent_prepare(const void* src, int src_stride, void* dst, int
 }
 
 // out[n, h, j] = (sum_k x[n, h, k] W[h, j, k]) * (gate ? sigmoid(gate[n, h * Nout + j]) : 1).
-// grid: (tiles of Nout, tiles of N, H).
-template <typename T>
+// grid: (tiles of Nout, tiles of N, H).  MFMA: the tile on the matrix cores (bfloat16, rows readable 16 bytes
+// at a time), else on the vector ALUs in fp32.
+template <bool MFMA, typename T>
 __global__ __launch_bounds__(256) void gemm_heads_kernel(const T* __restrict__ x, int x_row, int x_head,
                                                          const T* __restrict__ W, T* __restrict__ out, int o_row,
                                                          int o_head, const T* __restrict__ gate, int g_row, int N,
                                                          int Nout, int K) {
-  __shared__ TileFmaLds lds;
+  __shared__ TileLds lds;
   const int h = blockIdx.z;
   const int m0 = blockIdx.y * TF_T, n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (m0 + lr < N) ? x + (size_t)(m0 + lr) * x_row + (size_t)h * x_head : nullptr;
   const T* w_row = (n0 + lr < Nout) ? W + ((size_t)h * Nout + n0 + lr) * K : nullptr;
-  float acc[4][4];
-  tile_fma_64(a_row, w_row, K, acc, lds);
-  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty * 4 + i;
-    if (m >= N) continue;
+  tile_64<MFMA>(a_row, w_row, K, lds, [&](int i, int j0, const float* v) {
+    const int m = m0 + i;
+    if (m >= N) return;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int c = n0 + tx * 4 + j;
+      const int c = n0 + j0 + j;
       if (c >= Nout) continue;
-      float v = acc[i][j];
+      float y = v[j];
       if (gate) {
         const float g = to_float(gate[(size_t)m * g_row + (size_t)h * Nout + c]);
-        v = to_float(from_float<T>(v)) * (1.0f / (1.0f + expf(-g)));    // the product is stored first, as a tensor would be
+        y = to_float(from_float<T>(y)) * (1.0f / (1.0f + expf(-g)));    // the product is stored first, as a tensor would be
       }
-      out[(size_t)m * o_row + (size_t)h * o_head + c] = from_float<T>(v);
+      out[(size_t)m * o_row + (size_t)h * o_head + c] = from_float<T>(y);
     }
-  }
+  });
 }
 
 extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W, void* out, int o_row, int o_head,
@@ -109,12 +106,17 @@ extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W
   dim3 grid((Nout + TF_T - 1) / TF_T, (N + TF_T - 1) / TF_T, H);
   if (grid.y > 65535u || grid.z > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    gemm_heads_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)W, (float*)out,
-                                                       o_row, o_head, (const float*)gate, g_row, N, Nout, K);
+    gemm_heads_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)W,
+                                                              (float*)out, o_row, o_head, (const float*)gate, g_row,
+                                                              N, Nout, K);
+  else if (dtype == IA_BF16 && (K & 7) == 0 && tile_rows_aligned(x, x_row, x_head) && tile_rows_aligned(W, K))
+    gemm_heads_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+                                                              (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row,
+                                                              N, Nout, K);
   else if (dtype == IA_BF16)
-    gemm_heads_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
-                                                        (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
-                                                        Nout, K);
+    gemm_heads_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+                                                               (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row,
+                                                               N, Nout, K);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

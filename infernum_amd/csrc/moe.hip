@@ -111,35 +111,32 @@ __device__ __forceinline__ bool moe_tile(const int* __restrict__ offsets, int E,
 }
 
 // grid: (tiles of 2 * ff columns, ceil(P / 64) + E).  Wgu [E, 2 ff, W]: row 2 j the gate's row j, row 2 j + 1 up's.
-template <typename T>
+// MFMA: the tile on the matrix cores (bfloat16, rows readable 16 bytes at a time), else on the vector ALUs.
+template <bool MFMA, typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ Wgu,
                                                           T* __restrict__ y, const int* __restrict__ offsets,
                                                           const int* __restrict__ perm, int E, int top, int W,
                                                           int ff, float limit, float alpha) {
-  __shared__ TileFmaLds lds;
+  __shared__ TileLds lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
   const int n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (first + lr < last) ? x + (size_t)(perm[first + lr] / top) * W : nullptr;
   const T* w_row = (n0 + lr < 2 * ff) ? Wgu + ((size_t)e * 2 * ff + n0 + lr) * W : nullptr;
-  float acc[4][4];
-  tile_fma_64(a_row, w_row, W, acc, lds);
-  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int p = first + ty * 4 + i;
-    if (p >= last) continue;
+  tile_64<MFMA>(a_row, w_row, W, lds, [&](int i, int j0, const float* v) {
+    const int p = first + i;
+    if (p >= last) return;
 #pragma unroll
     for (int j = 0; j < 4; j += 2) {
-      const int c = n0 + tx * 4 + j;
+      const int c = n0 + j0 + j;
       if (c + 1 >= 2 * ff) continue;
       // both products are rounded as a stored tensor would be, then the activation in fp32
-      const float g = fminf(to_float(from_float<T>(acc[i][j])), limit);
-      const float u = fminf(fmaxf(to_float(from_float<T>(acc[i][j + 1])), -limit), limit);
+      const float g = fminf(to_float(from_float<T>(v[j])), limit);
+      const float u = fminf(fmaxf(to_float(from_float<T>(v[j + 1])), -limit), limit);
       y[(size_t)p * ff + (c >> 1)] = from_float<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
     }
-  }
+  });
 }
 
 extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int* offsets, const int* perm, int dtype,
@@ -149,11 +146,14 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
   dim3 grid((2 * ff + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
   if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    moe_gate_up_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets, perm,
-                                                        E, top, W, ff, limit, alpha);
+    moe_gate_up_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets,
+                                                               perm, E, top, W, ff, limit, alpha);
+  else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wgu, W))
+    moe_gate_up_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
+                                                               offsets, perm, E, top, W, ff, limit, alpha);
   else if (dtype == IA_BF16)
-    moe_gate_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
-                                                         perm, E, top, W, ff, limit, alpha);
+    moe_gate_up_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
+                                                                offsets, perm, E, top, W, ff, limit, alpha);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();
@@ -161,35 +161,31 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
 }
 
 // grid: (tiles of W columns, ceil(P / 64) + E).  Wd [E, W, ff]; parts [top, N, W] fp32.
-template <typename T>
+template <bool MFMA, typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ y, const T* __restrict__ Wd,
                                                        float* __restrict__ parts, const float* __restrict__ weights,
                                                        const int* __restrict__ offsets, const int* __restrict__ perm,
                                                        int E, int top, int N, int W, int ff) {
-  __shared__ TileFmaLds lds;
+  __shared__ TileLds lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
   const int n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (first + lr < last) ? y + (size_t)(first + lr) * ff : nullptr;
   const T* w_row = (n0 + lr < W) ? Wd + ((size_t)e * W + n0 + lr) * ff : nullptr;
-  float acc[4][4];
-  tile_fma_64(a_row, w_row, ff, acc, lds);
-  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int p = first + ty * 4 + i;
-    if (p >= last) continue;
+  tile_64<MFMA>(a_row, w_row, ff, lds, [&](int i, int j0, const float* v) {
+    const int p = first + i;
+    if (p >= last) return;
     const int pair = perm[p];
     const int token = pair / top, choice = pair - token * top;
     const float wt = weights[pair];
     float* o = parts + ((size_t)choice * N + token) * W;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int c = n0 + tx * 4 + j;
-      if (c < W) o[c] = to_float(from_float<T>(acc[i][j])) * wt;
+      const int c = n0 + j0 + j;
+      if (c < W) o[c] = to_float(from_float<T>(v[j])) * wt;
     }
-  }
+  });
 }
 
 extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const float* weights, const int* offsets,
@@ -200,11 +196,14 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
   dim3 grid((W + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
   if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    moe_down_kernel<float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets, perm,
-                                                     E, top, N, W, ff);
+    moe_down_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets,
+                                                            perm, E, top, N, W, ff);
+  else if (dtype == IA_BF16 && tile_rows_aligned(y, ff) && tile_rows_aligned(Wd, ff))
+    moe_down_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
+                                                            offsets, perm, E, top, N, W, ff);
   else if (dtype == IA_BF16)
-    moe_down_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
-                                                      perm, E, top, N, W, ff);
+    moe_down_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
+                                                             offsets, perm, E, top, N, W, ff);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();
