@@ -12,8 +12,29 @@ __global__ __launch_bounds__(256) void activation_kernel(const T* __restrict__ i
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
     const float z = to_float(in[i]);
     float y = z;
-    if (kind == IA_ACT_GELU_TANH) y = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    if (kind == IA_ACT_GELU_TANH) y = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));   // gelu_tanh_f below, same roundings
     out[i] = from_float<T>(y);
+  }
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// Eight bfloat16 values (16 bytes) a thread and pass.
+__global__ __launch_bounds__(256) void gelu_tanh_bf16x8_kernel(const uint4* __restrict__ in, uint4* __restrict__ out,
+                                                               size_t n8) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += stride) {
+    const uint4 v = in[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float lo = gelu_tanh_f(__uint_as_float(w[k] << 16)), hi = gelu_tanh_f(__uint_as_float(w[k] & 0xffff0000u));
+      o[k] = (uint32_t)float_to_bf16_bits(lo) | ((uint32_t)float_to_bf16_bits(hi) << 16);
+    }
+    out[i] = make_uint4(o[0], o[1], o[2], o[3]);
   }
 }
 
@@ -22,6 +43,13 @@ extern "C" int ia_activation(const void* in, void* out, int dtype, size_t n, int
   if (n == 0) return IA_OK;
   if (!in || !out) return IA_ERR_BAD_ARG;
   const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (dtype == IA_BF16 && (n & 7) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    const size_t n8 = n >> 3;
+    gelu_tanh_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256 < 65536 ? (n8 + 255) / 256 : 65536), 256, 0, stream>>>(
+        (const uint4*)in, (uint4*)out, n8);
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
   if (dtype == IA_F32)
     activation_kernel<float><<<grid, 256, 0, stream>>>((const float*)in, (float*)out, n, kind);
   else

@@ -96,6 +96,35 @@ __global__ __launch_bounds__(256) void gemm_heads_kernel(const T* __restrict__ x
   });
 }
 
+// The same on tiles of BM x 128 (tile_mfma_big): grid (tiles of 128 of Nout, tiles of BM of N, H).
+template <int BM>
+__global__ __launch_bounds__(256) void gemm_heads_big_kernel(const bf16_t* __restrict__ x, int x_row, int x_head,
+                                                             const bf16_t* __restrict__ W, bf16_t* __restrict__ out,
+                                                             int o_row, int o_head, const bf16_t* __restrict__ gate,
+                                                             int g_row, int N, int Nout, int K) {
+  __shared__ TileBigLds<BM> lds;
+  const int h = blockIdx.z;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * TB_N;
+  tile_mfma_big<BM>(
+      [&](int r) { return m0 + r < N ? x + (size_t)(m0 + r) * x_row + (size_t)h * x_head : nullptr; },
+      [&](int r) { return n0 + r < Nout ? W + ((size_t)h * Nout + n0 + r) * K : nullptr; }, K, lds,
+      [&](int i, int j0, const float* v) {
+        const int m = m0 + i;
+        if (m >= N) return;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = n0 + j0 + j;
+          if (c >= Nout) continue;
+          float y = v[j];
+          if (gate) {
+            const float g = to_float(gate[(size_t)m * g_row + (size_t)h * Nout + c]);
+            y = to_float(from_float<bf16_t>(y)) * (1.0f / (1.0f + expf(-g)));
+          }
+          out[(size_t)m * o_row + (size_t)h * o_head + c] = from_float<bf16_t>(y);
+        }
+      });
+}
+
 extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W, void* out, int o_row, int o_head,
                              const void* gate, int g_row, int dtype, int N, int H, int Nout, int K,
                              hipStream_t stream) {
@@ -109,10 +138,18 @@ extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W
     gemm_heads_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)W,
                                                               (float*)out, o_row, o_head, (const float*)gate, g_row,
                                                               N, Nout, K);
-  else if (dtype == IA_BF16 && (K & 7) == 0 && tile_rows_aligned(x, x_row, x_head) && tile_rows_aligned(W, K))
-    gemm_heads_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
-                                                              (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row,
-                                                              N, Nout, K);
+  else if (dtype == IA_BF16 && (K & 7) == 0 && tile_rows_aligned(x, x_row, x_head) && tile_rows_aligned(W, K)) {
+    const int bm = N >= 96 ? 128 : 32;
+    dim3 big((Nout + TB_N - 1) / TB_N, (N + bm - 1) / bm, H);
+    if (bm == 128)
+      gemm_heads_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+                                                          (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
+                                                          Nout, K);
+    else
+      gemm_heads_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+                                                         (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
+                                                         Nout, K);
+  }
   else if (dtype == IA_BF16)
     gemm_heads_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
                                                                (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row,

@@ -11,44 +11,64 @@
 #include "common.h"
 #include "tile_fma.h"
 
+// One wave a token: lane l holds the logits of experts l, l + 64, ...; `top` rounds of "the largest not taken yet"
+// (the lowest index among equals), each a maximum over the wave.
+#define RT_PER_LANE 16        // experts a lane holds: E <= 64 * RT_PER_LANE
 __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
                                                           const void* __restrict__ bias, int bias_dtype,
                                                           int* __restrict__ ids, float* __restrict__ weights, int N,
                                                           int E, int top) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (n >= N) return;
   const float* z = logits + (size_t)n * E;
-  float prev_v = INFINITY, first_v = 0.f, sum = 0.f;
-  int prev_i = -1;
+  float v[RT_PER_LANE];
+  unsigned taken = 0u;
+#pragma unroll
+  for (int c = 0; c < RT_PER_LANE; ++c) {
+    const int e = lane + 64 * c;
+    v[c] = e < E ? z[e] + (bias ? load_as_float(bias, bias_dtype, e) : 0.f) : -INFINITY;
+    if (e >= E) taken |= 1u << c;
+  }
+  float first_v = 0.f, sum = 0.f;
   for (int k = 0; k < top; ++k) {
     float best_v = -INFINITY;
-    int best_i = -1;
-    for (int e = 0; e < E; ++e) {
-      const float v = z[e] + (bias ? load_as_float(bias, bias_dtype, e) : 0.f);
-      const bool after = (v < prev_v) || (v == prev_v && e > prev_i);       // not chosen yet
-      if (after && (best_i < 0 || v > best_v)) { best_v = v; best_i = e; }
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int c = 0; c < RT_PER_LANE; ++c) {
+      const bool free_ = !((taken >> c) & 1u);
+      // a value that compares with nothing (NaN) counts as the smallest
+      const float x = (v[c] == v[c]) ? v[c] : -INFINITY;
+      if (free_ && (best_e == 0x7fffffff || x > best_v)) { best_v = x; best_e = lane + 64 * c; }
     }
-    if (best_i < 0) {          // values that compare with nothing (NaN): any expert not chosen yet, by index
-      best_i = prev_i + 1 < E ? prev_i + 1 : 0;
-      best_v = z[best_i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best_v, o, IA_WAVE);
+      const int oe = __shfl_xor(best_e, o, IA_WAVE);
+      if (oe != 0x7fffffff && (best_e == 0x7fffffff || ov > best_v || (ov == best_v && oe < best_e))) {
+        best_v = ov;
+        best_e = oe;
+      }
     }
+    if ((best_e & 63) == lane) taken |= 1u << (best_e >> 6);
     if (k == 0) first_v = best_v;
     const float w = expf(best_v - first_v);
-    ids[(size_t)n * top + k] = best_i;
-    weights[(size_t)n * top + k] = w;
     sum += w;
-    prev_v = best_v;
-    prev_i = best_i;
+    if (lane == 0) {
+      ids[(size_t)n * top + k] = best_e;
+      weights[(size_t)n * top + k] = w;
+    }
   }
   const float inv = 1.0f / sum;
-  for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] *= inv;
+  if (lane == 0)
+    for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] *= inv;
 }
 
 extern "C" int ia_router_topk(const float* logits, const void* bias, int bias_dtype, int* ids, float* weights, int N,
                               int E, int top, hipStream_t stream) {
   if (N < 0 || E <= 0 || top <= 0 || top > E) return IA_ERR_BAD_ARG;
+  if (E > 64 * RT_PER_LANE) return IA_ERR_UNSUPPORTED;
   if (N == 0) return IA_OK;
-  router_topk_kernel<<<(N + 255) / 256, 256, 0, stream>>>(logits, bias, bias_dtype, ids, weights, N, E, top);
+  router_topk_kernel<<<(N + 3) / 4, 256, 0, stream>>>(logits, bias, bias_dtype, ids, weights, N, E, top);
   IA_LAUNCH_CHECK();
   return IA_OK;
 }
@@ -91,17 +111,17 @@ extern "C" int ia_moe_sort(const int* ids, int* offsets, int* perm, int P, int E
   return IA_OK;
 }
 
-// Tile t of the launch (rows of 64 pairs, expert by expert): its expert and its first place in perm; false when
+// Tile t of the launch (`rows` pairs a tile, expert by expert): its expert and its first place in perm; false when
 // the launch has more tiles than the step needs.
 __device__ __forceinline__ bool moe_tile(const int* __restrict__ offsets, int E, int t, int& expert, int& first,
-                                         int& last) {
+                                         int& last, int rows = TF_T) {
   int seen = 0;
   for (int e = 0; e < E; ++e) {
     const int lo = offsets[e], hi = offsets[e + 1];
-    const int tiles = (hi - lo + TF_T - 1) / TF_T;
+    const int tiles = (hi - lo + rows - 1) / rows;
     if (t < seen + tiles) {
       expert = e;
-      first = lo + (t - seen) * TF_T;
+      first = lo + (t - seen) * rows;
       last = hi;
       return true;
     }
@@ -139,6 +159,36 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
   });
 }
 
+// The same on tiles of BM x 128 (tile_mfma_big): grid (tiles of 128 of the 2 ff columns, ceil(P / BM) + E).
+template <int BM>
+__global__ __launch_bounds__(256) void moe_gate_up_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wgu,
+                                                              bf16_t* __restrict__ y, const int* __restrict__ offsets,
+                                                              const int* __restrict__ perm, int E, int top, int W,
+                                                              int ff, float limit, float alpha) {
+  __shared__ TileBigLds<BM> lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
+  const int n0 = blockIdx.x * TB_N;
+  tile_mfma_big<BM>(
+      [&](int r) { return first + r < last ? x + (size_t)(perm[first + r] / top) * W : nullptr; },
+      [&](int r) { return n0 + r < 2 * ff ? Wgu + ((size_t)e * 2 * ff + n0 + r) * W : nullptr; }, W, lds,
+      [&](int i, int j0, const float* v) {
+        const int p = first + i;
+        if (p >= last) return;
+#pragma unroll
+        for (int j = 0; j < 4; j += 2) {
+          const int c = n0 + j0 + j;
+          if (c + 1 >= 2 * ff) continue;
+          const float g = fminf(to_float(from_float<bf16_t>(v[j])), limit);
+          const float u = fminf(fmaxf(to_float(from_float<bf16_t>(v[j + 1])), -limit), limit);
+          y[(size_t)p * ff + (c >> 1)] = from_float<bf16_t>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f));
+        }
+      });
+}
+
+// Rows a tile of the experts' products takes: 128 where an expert has some tens of pairs on average, else 32.
+static inline int moe_tile_rows(int P, int E) { return (long)P >= 48L * E ? 128 : 32; }
+
 extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int* offsets, const int* perm, int dtype,
                               int P, int E, int top, int W, int ff, float limit, float alpha, hipStream_t stream) {
   if (P < 0 || E <= 0 || top <= 0 || W <= 0 || ff <= 0) return IA_ERR_BAD_ARG;
@@ -148,9 +198,17 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
   if (dtype == IA_F32)
     moe_gate_up_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets,
                                                                perm, E, top, W, ff, limit, alpha);
-  else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wgu, W))
-    moe_gate_up_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
-                                                               offsets, perm, E, top, W, ff, limit, alpha);
+  else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wgu, W)) {
+    const int bm = moe_tile_rows(P, E);
+    dim3 big((2 * ff + TB_N - 1) / TB_N, (P + bm - 1) / bm + E);
+    if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
+    if (bm == 128)
+      moe_gate_up_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
+                                                           perm, E, top, W, ff, limit, alpha);
+    else
+      moe_gate_up_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
+                                                          perm, E, top, W, ff, limit, alpha);
+  }
   else if (dtype == IA_BF16)
     moe_gate_up_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
                                                                 offsets, perm, E, top, W, ff, limit, alpha);
@@ -188,6 +246,33 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ y, 
   });
 }
 
+template <int BM>
+__global__ __launch_bounds__(256) void moe_down_big_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ Wd,
+                                                           float* __restrict__ parts, const float* __restrict__ weights,
+                                                           const int* __restrict__ offsets, const int* __restrict__ perm,
+                                                           int E, int top, int N, int W, int ff) {
+  __shared__ TileBigLds<BM> lds;
+  int e, first, last;
+  if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
+  const int n0 = blockIdx.x * TB_N;
+  tile_mfma_big<BM>(
+      [&](int r) { return first + r < last ? y + (size_t)(first + r) * ff : nullptr; },
+      [&](int r) { return n0 + r < W ? Wd + ((size_t)e * W + n0 + r) * ff : nullptr; }, ff, lds,
+      [&](int i, int j0, const float* v) {
+        const int p = first + i;
+        if (p >= last) return;
+        const int pair = perm[p];
+        const int token = pair / top, choice = pair - token * top;
+        const float wt = weights[pair];
+        float* o = parts + ((size_t)choice * N + token) * W;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int c = n0 + j0 + j;
+          if (c < W) o[c] = to_float(from_float<bf16_t>(v[j])) * wt;
+        }
+      });
+}
+
 extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const float* weights, const int* offsets,
                            const int* perm, int dtype, int N, int E, int top, int W, int ff, hipStream_t stream) {
   if (N < 0 || E <= 0 || top <= 0 || W <= 0 || ff <= 0) return IA_ERR_BAD_ARG;
@@ -198,9 +283,17 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
   if (dtype == IA_F32)
     moe_down_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets,
                                                             perm, E, top, N, W, ff);
-  else if (dtype == IA_BF16 && tile_rows_aligned(y, ff) && tile_rows_aligned(Wd, ff))
-    moe_down_kernel<true, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
-                                                            offsets, perm, E, top, N, W, ff);
+  else if (dtype == IA_BF16 && tile_rows_aligned(y, ff) && tile_rows_aligned(Wd, ff)) {
+    const int bm = moe_tile_rows(P, E);
+    dim3 big((W + TB_N - 1) / TB_N, (P + bm - 1) / bm + E);
+    if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
+    if (bm == 128)
+      moe_down_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
+                                                        perm, E, top, N, W, ff);
+    else
+      moe_down_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
+                                                       perm, E, top, N, W, ff);
+  }
   else if (dtype == IA_BF16)
     moe_down_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
                                                              offsets, perm, E, top, N, W, ff);

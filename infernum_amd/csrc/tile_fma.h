@@ -163,3 +163,87 @@ __device__ __forceinline__ void tile_64(const T* __restrict__ a_row, const T* __
 __host__ __device__ inline bool tile_rows_aligned(const void* p, long stride, long stride2 = 0) {
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (stride & 7) == 0 && (stride2 & 7) == 0;
 }
+
+// ---- a larger tile on the matrix cores: BM rows of A (128, or 32 for steps of few rows) x 128 rows of W ------------
+// 256 threads = 4 waves, 2 x 2 over the tile at BM = 128 (64 x 64 a wave: 4 x 4 accumulators) and 1 x 4 at BM = 32
+// (32 x 32 a wave).  K is walked in steps of 32 through two LDS stages: the global loads of step i + 1 are issued
+// before the matrix instructions of step i and stored to the other stage after them, one barrier a step.  Operand
+// fragments and the result's layout are those of tile_mfma_64: a lane ends with four consecutive columns of one row.
+// `a_row(r)` / `w_row(r)`: row r of the tile's A / W (16-byte aligned, K a multiple of 8), or nullptr.
+#define TB_KS 32
+#define TB_LD 40
+#define TB_N 128
+
+template <int BM>
+struct TileBigLds {
+  uint16_t a[2][BM][TB_LD];
+  uint16_t w[2][TB_N][TB_LD];
+};
+
+template <int BM, typename ARow, typename WRow, typename Emit>
+__device__ __forceinline__ void tile_mfma_big(ARow a_row, WRow w_row, int K, TileBigLds<BM>& lds, Emit emit) {
+  static_assert(BM == 128 || BM == 32, "tiles of 128 or 32 rows");
+  constexpr int WM = BM == 128 ? 2 : 1, WN = 4 / WM;           // waves along the rows and the columns
+  constexpr int MT = BM / WM / 16, NT = TB_N / WN / 16;       // 16 x 16 tiles a wave
+  constexpr int ALOADS = BM >= 64 ? BM / 64 : 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, q = lane >> 4;
+  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (TB_N / WN);
+  const int lr = tid >> 2, lk = (tid & 3) * 8;
+  const bf16_t* ap[ALOADS];
+  const bf16_t* wp[2];
+#pragma unroll
+  for (int s = 0; s < ALOADS; ++s) ap[s] = (lr + 64 * s < BM) ? a_row(lr + 64 * s) : nullptr;
+#pragma unroll
+  for (int s = 0; s < 2; ++s) wp[s] = w_row(lr + 64 * s);
+  tm_f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = tm_f32x4{0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  uint4 ra[ALOADS], rw[2];
+  auto fetch = [&](int k0) {
+    const int k = k0 + lk;
+#pragma unroll
+    for (int s = 0; s < ALOADS; ++s) ra[s] = (ap[s] && k < K) ? *reinterpret_cast<const uint4*>(ap[s] + k) : zero;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) rw[s] = (wp[s] && k < K) ? *reinterpret_cast<const uint4*>(wp[s] + k) : zero;
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int s = 0; s < ALOADS; ++s)
+      if (lr + 64 * s < BM) *reinterpret_cast<uint4*>(&lds.a[buf][lr + 64 * s][lk]) = ra[s];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) *reinterpret_cast<uint4*>(&lds.w[buf][lr + 64 * s][lk]) = rw[s];
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  const int steps = (K + TB_KS - 1) / TB_KS;
+  for (int i = 0; i < steps; ++i) {
+    const int buf = i & 1;
+    const bool more = i + 1 < steps;
+    if (more) fetch((i + 1) * TB_KS);
+    uint4 wf[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wf[nt] = *reinterpret_cast<const uint4*>(&lds.w[buf][wn0 + 16 * nt + r][q * 8]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const uint4 af = *reinterpret_cast<const uint4*>(&lds.a[buf][wm0 + 16 * mt + r][q * 8]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tm_bf16x8, wf[nt]),
+                                                              __builtin_bit_cast(tm_bf16x8, af), acc[mt][nt], 0, 0, 0);
+    }
+    if (more) stage(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float v[4] = {acc[mt][nt][0], acc[mt][nt][1], acc[mt][nt][2], acc[mt][nt][3]};
+      emit(wm0 + 16 * mt + r, wn0 + 16 * nt + 4 * q, v);
+    }
+}
