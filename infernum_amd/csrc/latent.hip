@@ -106,8 +106,8 @@ __global__ __launch_bounds__(256) void gemm_heads_big_kernel(const bf16_t* __res
   const int h = blockIdx.z;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * TB_N;
   tile_mfma_big<BM>(
-      [&](int r) { return m0 + r < N ? x + (size_t)(m0 + r) * x_row + (size_t)h * x_head : nullptr; },
-      [&](int r) { return n0 + r < Nout ? W + ((size_t)h * Nout + n0 + r) * K : nullptr; }, K, lds,
+      [&](int r) { return x + (size_t)(m0 + r) * x_row + (size_t)h * x_head; },
+      [&](int r) { return W + ((size_t)h * Nout + n0 + r) * K; }, N - m0, Nout - n0, K, lds,
       [&](int i, int j0, const float* v) {
         const int m = m0 + i;
         if (m >= N) return;

@@ -170,8 +170,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_big_kernel(const bf16_t* __re
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
   const int n0 = blockIdx.x * TB_N;
   tile_mfma_big<BM>(
-      [&](int r) { return first + r < last ? x + (size_t)(perm[first + r] / top) * W : nullptr; },
-      [&](int r) { return n0 + r < 2 * ff ? Wgu + ((size_t)e * 2 * ff + n0 + r) * W : nullptr; }, W, lds,
+      [&](int r) { return x + (size_t)(perm[first + r] / top) * W; },
+      [&](int r) { return Wgu + ((size_t)e * 2 * ff + n0 + r) * W; }, last - first, 2 * ff - n0, W, lds,
       [&](int i, int j0, const float* v) {
         const int p = first + i;
         if (p >= last) return;
@@ -256,8 +256,8 @@ __global__ __launch_bounds__(256) void moe_down_big_kernel(const bf16_t* __restr
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
   const int n0 = blockIdx.x * TB_N;
   tile_mfma_big<BM>(
-      [&](int r) { return first + r < last ? y + (size_t)(first + r) * ff : nullptr; },
-      [&](int r) { return n0 + r < W ? Wd + ((size_t)e * W + n0 + r) * ff : nullptr; }, ff, lds,
+      [&](int r) { return y + (size_t)(first + r) * ff; },
+      [&](int r) { return Wd + ((size_t)e * W + n0 + r) * ff; }, last - first, W - n0, ff, lds,
       [&](int i, int j0, const float* v) {
         const int p = first + i;
         if (p >= last) return;

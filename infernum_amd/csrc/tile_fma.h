@@ -166,77 +166,103 @@ __host__ __device__ inline bool tile_rows_aligned(const void* p, long stride, lo
 
 // ---- a larger tile on the matrix cores: BM rows of A (128, or 32 for steps of few rows) x 128 rows of W ------------
 // 256 threads = 4 waves, 2 x 2 over the tile at BM = 128 (64 x 64 a wave: 4 x 4 accumulators) and 1 x 4 at BM = 32
-// (32 x 32 a wave).  K is walked in steps of 32 through two LDS stages: the global loads of step i + 1 are issued
-// before the matrix instructions of step i and stored to the other stage after them, one barrier a step.  Operand
+// (32 x 32 a wave).  K is walked in steps of 64 through one LDS stage; the global loads run two steps ahead of the
+// matrix instructions in two sets of registers (the loads of step i + 2 are issued before the matrix instructions
+// of step i and stored to LDS after those of step i + 1), every load unconditional so that a wait for the older
+// set leaves the newer in flight: a row that the tile does not have is read from the tile's first row (its sums
+// are never handed on), and values of k past K are read from the row's end and set to zero by a select.  Operand
 // fragments and the result's layout are those of tile_mfma_64: a lane ends with four consecutive columns of one row.
-// `a_row(r)` / `w_row(r)`: row r of the tile's A / W (16-byte aligned, K a multiple of 8), or nullptr.
-#define TB_KS 32
-#define TB_LD 40
+// `a_row(r)` / `w_row(r)`: row r of the tile's A / W (16-byte aligned, K a multiple of 8 and at least 8); row 0
+// always exists.
+#define TB_KS 64
+#define TB_LD 72
 #define TB_N 128
 
 template <int BM>
 struct TileBigLds {
-  uint16_t a[2][BM][TB_LD];
-  uint16_t w[2][TB_N][TB_LD];
+  uint16_t a[BM][TB_LD];
+  uint16_t w[TB_N][TB_LD];
 };
 
 template <int BM, typename ARow, typename WRow, typename Emit>
-__device__ __forceinline__ void tile_mfma_big(ARow a_row, WRow w_row, int K, TileBigLds<BM>& lds, Emit emit) {
+__device__ __forceinline__ void tile_mfma_big(ARow a_row, WRow w_row, int a_rows, int w_rows, int K,
+                                              TileBigLds<BM>& lds, Emit emit) {
   static_assert(BM == 128 || BM == 32, "tiles of 128 or 32 rows");
   constexpr int WM = BM == 128 ? 2 : 1, WN = 4 / WM;           // waves along the rows and the columns
   constexpr int MT = BM / WM / 16, NT = TB_N / WN / 16;       // 16 x 16 tiles a wave
-  constexpr int ALOADS = BM >= 64 ? BM / 64 : 1;
+  constexpr int AR = BM / 32, WR = TB_N / 32;                 // rows of A and of W that a thread loads a step
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
   const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (TB_N / WN);
-  const int lr = tid >> 2, lk = (tid & 3) * 8;
-  const bf16_t* ap[ALOADS];
-  const bf16_t* wp[2];
+  const int lr = tid >> 3, lk = (tid & 7) * 8;                // 8 threads read a row's 64 values of k
+  const bf16_t* ap[AR];
+  const bf16_t* wp[WR];
 #pragma unroll
-  for (int s = 0; s < ALOADS; ++s) ap[s] = (lr + 64 * s < BM) ? a_row(lr + 64 * s) : nullptr;
+  for (int s = 0; s < AR; ++s) ap[s] = a_row(lr + 32 * s < a_rows ? lr + 32 * s : 0);
 #pragma unroll
-  for (int s = 0; s < 2; ++s) wp[s] = w_row(lr + 64 * s);
+  for (int s = 0; s < WR; ++s) wp[s] = w_row(lr + 32 * s < w_rows ? lr + 32 * s : 0);
   tm_f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = tm_f32x4{0.f, 0.f, 0.f, 0.f};
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-  uint4 ra[ALOADS], rw[2];
-  auto fetch = [&](int k0) {
+  uint4 ra[2][AR], rw[2][WR];
+  auto fetch = [&](int k0, uint4 (&xa)[AR], uint4 (&xw)[WR]) {
     const int k = k0 + lk;
+    const int kc = k < K ? k : K - 8;                          // stays inside the row
 #pragma unroll
-    for (int s = 0; s < ALOADS; ++s) ra[s] = (ap[s] && k < K) ? *reinterpret_cast<const uint4*>(ap[s] + k) : zero;
+    for (int s = 0; s < AR; ++s) xa[s] = *reinterpret_cast<const uint4*>(ap[s] + kc);
 #pragma unroll
-    for (int s = 0; s < 2; ++s) rw[s] = (wp[s] && k < K) ? *reinterpret_cast<const uint4*>(wp[s] + k) : zero;
-  };
-  auto stage = [&](int buf) {
+    for (int s = 0; s < WR; ++s) xw[s] = *reinterpret_cast<const uint4*>(wp[s] + kc);
+    if (k >= K) {
 #pragma unroll
-    for (int s = 0; s < ALOADS; ++s)
-      if (lr + 64 * s < BM) *reinterpret_cast<uint4*>(&lds.a[buf][lr + 64 * s][lk]) = ra[s];
+      for (int s = 0; s < AR; ++s) xa[s] = zero;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) *reinterpret_cast<uint4*>(&lds.w[buf][lr + 64 * s][lk]) = rw[s];
-  };
-  fetch(0);
-  stage(0);
-  __syncthreads();
-  const int steps = (K + TB_KS - 1) / TB_KS;
-  for (int i = 0; i < steps; ++i) {
-    const int buf = i & 1;
-    const bool more = i + 1 < steps;
-    if (more) fetch((i + 1) * TB_KS);
-    uint4 wf[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) wf[nt] = *reinterpret_cast<const uint4*>(&lds.w[buf][wn0 + 16 * nt + r][q * 8]);
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const uint4 af = *reinterpret_cast<const uint4*>(&lds.a[buf][wm0 + 16 * mt + r][q * 8]);
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tm_bf16x8, wf[nt]),
-                                                              __builtin_bit_cast(tm_bf16x8, af), acc[mt][nt], 0, 0, 0);
+      for (int s = 0; s < WR; ++s) xw[s] = zero;
     }
-    if (more) stage(buf ^ 1);
+  };
+  auto stage = [&](const uint4 (&xa)[AR], const uint4 (&xw)[WR]) {
+#pragma unroll
+    for (int s = 0; s < AR; ++s) *reinterpret_cast<uint4*>(&lds.a[lr + 32 * s][lk]) = xa[s];
+#pragma unroll
+    for (int s = 0; s < WR; ++s) *reinterpret_cast<uint4*>(&lds.w[lr + 32 * s][lk]) = xw[s];
+  };
+  auto multiply = [&]() {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 wf[NT];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) wf[nt] = *reinterpret_cast<const uint4*>(&lds.w[wn0 + 16 * nt + r][q * 8 + 32 * h]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const uint4 af = *reinterpret_cast<const uint4*>(&lds.a[wm0 + 16 * mt + r][q * 8 + 32 * h]);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tm_bf16x8, wf[nt]),
+                                                                __builtin_bit_cast(tm_bf16x8, af), acc[mt][nt], 0, 0, 0);
+      }
+    }
+  };
+  const int steps = (K + TB_KS - 1) / TB_KS;
+  fetch(0, ra[0], rw[0]);
+  fetch(TB_KS, ra[1], rw[1]);                                  // past K: zeros
+  stage(ra[0], rw[0]);
+  __syncthreads();
+  for (int i = 0; i < steps; i += 2) {
+    // step i: LDS holds it; set 0 is free for step i + 2, set 1 holds step i + 1
+    fetch((i + 2) * TB_KS, ra[0], rw[0]);
+    multiply();
+    __syncthreads();
+    if (i + 1 >= steps) break;
+    stage(ra[1], rw[1]);
+    __syncthreads();
+    // step i + 1
+    fetch((i + 3) * TB_KS, ra[1], rw[1]);
+    multiply();
+    __syncthreads();
+    if (i + 2 >= steps) break;
+    stage(ra[0], rw[0]);
     __syncthreads();
   }
 #pragma unroll
