@@ -66,20 +66,20 @@ extern "C" int ia_latent_prepare(const void* src, int src_stride, void* dst, int
 }
 
 // out[n, h, j] = (sum_k x[n, h, k] W[h, j, k]) * (gate ? sigmoid(gate[n, h * Nout + j]) : 1).
-// grid: (tiles of Nout, tiles of N, H).  MFMA: the tile on the matrix cores (bfloat16, rows readable 16 bytes
-// at a time), else on the vector ALUs in fp32.
-template <bool MFMA, typename T>
+// grid: (tiles of Nout, tiles of N, H).  On the vector ALUs in fp32: the 32-bit path, and bfloat16 rows that
+// cannot be read 16 bytes at a time.
+template <typename T>
 __global__ __launch_bounds__(256) void gemm_heads_kernel(const T* __restrict__ x, int x_row, int x_head,
                                                          const T* __restrict__ W, T* __restrict__ out, int o_row,
                                                          int o_head, const T* __restrict__ gate, int g_row, int N,
                                                          int Nout, int K) {
-  __shared__ TileLds lds;
+  __shared__ TileFmaLds lds;
   const int h = blockIdx.z;
   const int m0 = blockIdx.y * TF_T, n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (m0 + lr < N) ? x + (size_t)(m0 + lr) * x_row + (size_t)h * x_head : nullptr;
   const T* w_row = (n0 + lr < Nout) ? W + ((size_t)h * Nout + n0 + lr) * K : nullptr;
-  tile_64<MFMA>(a_row, w_row, K, lds, [&](int i, int j0, const float* v) {
+  tile_64(a_row, w_row, K, lds, [&](int i, int j0, const float* v) {
     const int m = m0 + i;
     if (m >= N) return;
 #pragma unroll
@@ -135,7 +135,7 @@ extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W
   dim3 grid((Nout + TF_T - 1) / TF_T, (N + TF_T - 1) / TF_T, H);
   if (grid.y > 65535u || grid.z > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    gemm_heads_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)W,
+    gemm_heads_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_row, x_head, (const float*)W,
                                                               (float*)out, o_row, o_head, (const float*)gate, g_row,
                                                               N, Nout, K);
   else if (dtype == IA_BF16 && (K & 7) == 0 && tile_rows_aligned(x, x_row, x_head) && tile_rows_aligned(W, K)) {
@@ -151,7 +151,7 @@ extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W
                                                          Nout, K);
   }
   else if (dtype == IA_BF16)
-    gemm_heads_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+    gemm_heads_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
                                                                (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row,
                                                                N, Nout, K);
   else

@@ -131,20 +131,20 @@ __device__ __forceinline__ bool moe_tile(const int* __restrict__ offsets, int E,
 }
 
 // grid: (tiles of 2 * ff columns, ceil(P / 64) + E).  Wgu [E, 2 ff, W]: row 2 j the gate's row j, row 2 j + 1 up's.
-// MFMA: the tile on the matrix cores (bfloat16, rows readable 16 bytes at a time), else on the vector ALUs.
-template <bool MFMA, typename T>
+// On the vector ALUs in fp32: the 32-bit path, and bfloat16 rows that cannot be read 16 bytes at a time.
+template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ x, const T* __restrict__ Wgu,
                                                           T* __restrict__ y, const int* __restrict__ offsets,
                                                           const int* __restrict__ perm, int E, int top, int W,
                                                           int ff, float limit, float alpha) {
-  __shared__ TileLds lds;
+  __shared__ TileFmaLds lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
   const int n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (first + lr < last) ? x + (size_t)(perm[first + lr] / top) * W : nullptr;
   const T* w_row = (n0 + lr < 2 * ff) ? Wgu + ((size_t)e * 2 * ff + n0 + lr) * W : nullptr;
-  tile_64<MFMA>(a_row, w_row, W, lds, [&](int i, int j0, const float* v) {
+  tile_64(a_row, w_row, W, lds, [&](int i, int j0, const float* v) {
     const int p = first + i;
     if (p >= last) return;
 #pragma unroll
@@ -196,7 +196,7 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
   dim3 grid((2 * ff + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
   if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    moe_gate_up_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets,
+    moe_gate_up_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (const float*)Wgu, (float*)y, offsets,
                                                                perm, E, top, W, ff, limit, alpha);
   else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wgu, W)) {
     const int bm = moe_tile_rows(P, E);
@@ -210,7 +210,7 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
                                                           perm, E, top, W, ff, limit, alpha);
   }
   else if (dtype == IA_BF16)
-    moe_gate_up_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
+    moe_gate_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y,
                                                                 offsets, perm, E, top, W, ff, limit, alpha);
   else
     return IA_ERR_BAD_ARG;
@@ -219,19 +219,19 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
 }
 
 // grid: (tiles of W columns, ceil(P / 64) + E).  Wd [E, W, ff]; parts [top, N, W] fp32.
-template <bool MFMA, typename T>
+template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ y, const T* __restrict__ Wd,
                                                        float* __restrict__ parts, const float* __restrict__ weights,
                                                        const int* __restrict__ offsets, const int* __restrict__ perm,
                                                        int E, int top, int N, int W, int ff) {
-  __shared__ TileLds lds;
+  __shared__ TileFmaLds lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last)) return;
   const int n0 = blockIdx.x * TF_T;
   const int lr = threadIdx.x >> 2;
   const T* a_row = (first + lr < last) ? y + (size_t)(first + lr) * ff : nullptr;
   const T* w_row = (n0 + lr < W) ? Wd + ((size_t)e * W + n0 + lr) * ff : nullptr;
-  tile_64<MFMA>(a_row, w_row, ff, lds, [&](int i, int j0, const float* v) {
+  tile_64(a_row, w_row, ff, lds, [&](int i, int j0, const float* v) {
     const int p = first + i;
     if (p >= last) return;
     const int pair = perm[p];
@@ -281,7 +281,7 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
   dim3 grid((W + TF_T - 1) / TF_T, (P + TF_T - 1) / TF_T + E);
   if (grid.y > 65535u) return IA_ERR_UNSUPPORTED;
   if (dtype == IA_F32)
-    moe_down_kernel<false, float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets,
+    moe_down_kernel<float><<<grid, 256, 0, stream>>>((const float*)y, (const float*)Wd, parts, weights, offsets,
                                                             perm, E, top, N, W, ff);
   else if (dtype == IA_BF16 && tile_rows_aligned(y, ff) && tile_rows_aligned(Wd, ff)) {
     const int bm = moe_tile_rows(P, E);
@@ -295,7 +295,7 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
                                                        perm, E, top, N, W, ff);
   }
   else if (dtype == IA_BF16)
-    moe_down_kernel<false, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
+    moe_down_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights,
                                                              offsets, perm, E, top, N, W, ff);
   else
     return IA_ERR_BAD_ARG;

@@ -53,6 +53,89 @@ __global__ __launch_bounds__(NB_NT) void norm_add_kernel(float* __restrict__ h, 
   }
 }
 
+// Rows of a multiple of 4 values up to NT * 4 * NV: every thread keeps its pieces of the row in registers, read 16
+// (or 8) bytes at a time with the loads of all parts of a piece in flight together; one pass over memory.
+__device__ __forceinline__ float4 nb_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 nb_load4(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                     __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void nb_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void nb_store4(bf16_t* p, float4 v) {
+  uint2 u;
+  u.x = (uint32_t)float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16);
+  u.y = (uint32_t)float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename TD, typename TX, int NT, int NV>
+__global__ __launch_bounds__(NT) void norm_add_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                          int splits, size_t split_stride,
+                                                          const void* __restrict__ w, int w_dtype,
+                                                          TX* __restrict__ x, int H, float eps) {
+  __shared__ float red[NT / 64];
+  const int row = blockIdx.x;
+  const TD* dr = delta + (size_t)row * H;
+  float* hr = h + (size_t)row * H;
+  float4 d[NV], hv[NV], g[NV];
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    d[c] = hv[c] = g[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < H) {
+      hv[c] = nb_load4(hr + i);
+      g[c] = w_dtype == IA_F32 ? nb_load4((const float*)w + i) : nb_load4((const bf16_t*)w + i);
+      d[c] = nb_load4(dr + i);
+    }
+  }
+#pragma clang loop unroll_count(4)
+  for (int k = 1; k < splits; ++k) {                 // the parts in the order of their index
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+      const int i = (threadIdx.x + c * NT) * 4;
+      if (i < H) {
+        const float4 p = nb_load4(dr + k * split_stride + i);
+        d[c].x += p.x; d[c].y += p.y; d[c].z += p.z; d[c].w += p.w;
+      }
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NV; ++c)
+    ss += __builtin_fmaf(d[c].x, d[c].x, d[c].y * d[c].y) + __builtin_fmaf(d[c].z, d[c].z, d[c].w * d[c].w);
+  ss = block_sum<NT>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+  for (int c = 0; c < NV; ++c) {
+    const int i = (threadIdx.x + c * NT) * 4;
+    if (i < H) {
+      const float4 s = make_float4(hv[c].x + d[c].x * inv * g[c].x, hv[c].y + d[c].y * inv * g[c].y,
+                                   hv[c].z + d[c].z * inv * g[c].z, hv[c].w + d[c].w * inv * g[c].w);
+      nb_store4(hr + i, s);
+      if (x) nb_store4(x + (size_t)row * H + i, s);
+    }
+  }
+}
+
+template <typename TD, typename TX>
+static void launch_norm_add(float* h, const void* delta, int splits, size_t stride, const void* w, int w_dtype, void* x,
+                            int N, int H, float eps, hipStream_t stream) {
+  const TD* d = (const TD*)delta;
+  TX* xo = (TX*)x;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(delta) |
+                         reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15) == 0 &&
+                       (stride & 3) == 0;
+  if ((H & 3) == 0 && aligned && H <= 256 * 4)
+    norm_add_vec_kernel<TD, TX, 256, 1><<<N, 256, 0, stream>>>(h, d, splits, stride, w, w_dtype, xo, H, eps);
+  else if ((H & 3) == 0 && aligned && H <= 1024 * 4)      // the kernel follows from H alone: a row's sums are taken
+    norm_add_vec_kernel<TD, TX, 1024, 1><<<N, 1024, 0, stream>>>(h, d, splits, stride, w, w_dtype, xo, H, eps);   // in one order
+  else if ((H & 3) == 0 && aligned && H <= 1024 * 4 * 4)
+    norm_add_vec_kernel<TD, TX, 1024, 4><<<N, 1024, 0, stream>>>(h, d, splits, stride, w, w_dtype, xo, H, eps);
+  else
+    norm_add_kernel<TD, TX><<<N, NB_NT, 0, stream>>>(h, d, splits, stride, w, w_dtype, xo, H, eps);
+}
+
 // delta_dtype: type of delta (IA_F32 for partial sums); act_dtype: type of x.  delta is [splits, delta_rows, H].
 extern "C" int ia_norm_add(float* h, const void* delta, int delta_dtype, int splits, int delta_rows, const void* w,
                            int w_dtype, void* x, int act_dtype, int N, int H, float eps, hipStream_t stream) {
@@ -60,14 +143,11 @@ extern "C" int ia_norm_add(float* h, const void* delta, int delta_dtype, int spl
   if (N == 0) return IA_OK;
   const size_t stride = (size_t)delta_rows * H;
   if (delta_dtype == IA_F32 && act_dtype == IA_F32)
-    norm_add_kernel<float, float><<<N, NB_NT, 0, stream>>>(h, (const float*)delta, splits, stride, w, w_dtype,
-                                                           (float*)x, H, eps);
+    launch_norm_add<float, float>(h, delta, splits, stride, w, w_dtype, x, N, H, eps, stream);
   else if (delta_dtype == IA_BF16 && act_dtype == IA_BF16)
-    norm_add_kernel<bf16_t, bf16_t><<<N, NB_NT, 0, stream>>>(h, (const bf16_t*)delta, splits, stride, w, w_dtype,
-                                                             (bf16_t*)x, H, eps);
+    launch_norm_add<bf16_t, bf16_t>(h, delta, splits, stride, w, w_dtype, x, N, H, eps, stream);
   else if (delta_dtype == IA_F32 && act_dtype == IA_BF16)
-    norm_add_kernel<float, bf16_t><<<N, NB_NT, 0, stream>>>(h, (const float*)delta, splits, stride, w, w_dtype,
-                                                            (bf16_t*)x, H, eps);
+    launch_norm_add<float, bf16_t>(h, delta, splits, stride, w, w_dtype, x, N, H, eps, stream);
   else
     return IA_ERR_BAD_ARG;
   IA_LAUNCH_CHECK();

@@ -69,93 +69,15 @@ __device__ __forceinline__ void tile_fma_64(const TA* __restrict__ a_row, const 
   }
 }
 
-// ---- the same tile on the matrix cores, for bfloat16 operands ---------------------------------------------------
-// 256 threads = 4 waves; K is walked in steps of 64 through LDS (rows padded to 72 values so that the 16-byte
-// reads of a wave's lanes spread over the banks), the next step's global loads in flight while this one's matrix
-// instructions run.  v_mfma_f32_16x16x32_bf16 with 16 rows of W as its first operand and 16 rows of A as its
-// second: lane (r = lane % 16, q = lane / 16) ends with D[column 4 q + e of W's 16][row r of A's 16], e = 0..3, so
-// a lane holds four consecutive columns of one row of the result, as a thread of the fp32 tile above does.  Wave w
-// takes columns 16 w .. 16 w + 15 of the tile for all 64 rows.  Rows of A and W must be 16-byte aligned and K a
-// multiple of 8 (values of k past K are taken as zero).  Every element is summed in an order that depends on K
-// alone.
-#define TM_KS 64
-#define TM_LD 72
-
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 tm_bf16x8;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float tm_f32x4;
-
-struct TileMfmaLds {
-  uint16_t a[TF_T][TM_LD];
-  uint16_t w[TF_T][TM_LD];
-};
-
-union TileLds {
-  TileFmaLds fma;
-  TileMfmaLds mfma;
-};
-
-// `a_row`, `w_row`: this thread's row (tid >> 2 of the tile) of A and of W, or nullptr.  acc[mt][e]: row
-// mt * 16 + (lane % 16), column 16 * wave + 4 * (lane / 16) + e.
-__device__ __forceinline__ void tile_mfma_64(const bf16_t* __restrict__ a_row, const bf16_t* __restrict__ w_row,
-                                             int K, tm_f32x4 (&acc)[4], TileMfmaLds& lds) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, q = lane >> 4;
-  const int lr = tid >> 2, lk = (tid & 3) * 8;          // this thread loads k = lk .. lk + 7 and lk + 32 .. lk + 39
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) acc[mt] = tm_f32x4{0.f, 0.f, 0.f, 0.f};
-  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-  uint4 ra[2], rw[2];
-  auto fetch = [&](int k0) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const int k = k0 + lk + 32 * s;
-      ra[s] = (a_row && k < K) ? *reinterpret_cast<const uint4*>(a_row + k) : zero;
-      rw[s] = (w_row && k < K) ? *reinterpret_cast<const uint4*>(w_row + k) : zero;
-    }
-  };
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += TM_KS) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      *reinterpret_cast<uint4*>(&lds.a[lr][lk + 32 * s]) = ra[s];
-      *reinterpret_cast<uint4*>(&lds.w[lr][lk + 32 * s]) = rw[s];
-    }
-    __syncthreads();
-    if (k0 + TM_KS < K) fetch(k0 + TM_KS);
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const uint4 wf = *reinterpret_cast<const uint4*>(&lds.w[16 * wave + r][q * 8 + 32 * s]);
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const uint4 af = *reinterpret_cast<const uint4*>(&lds.a[16 * mt + r][q * 8 + 32 * s]);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(tm_bf16x8, wf),
-                                                          __builtin_bit_cast(tm_bf16x8, af), acc[mt], 0, 0, 0);
-      }
-    }
-    __syncthreads();
-  }
-}
-
-// One tile by either way, handed to `emit(row of the tile, first of four consecutive columns, the four sums)`.
-template <bool MFMA, typename T, typename Emit>
+// The fp32 tile, handed to `emit(row of the tile, first of four consecutive columns, the four sums)`.
+template <typename T, typename Emit>
 __device__ __forceinline__ void tile_64(const T* __restrict__ a_row, const T* __restrict__ w_row, int K,
-                                        TileLds& lds, Emit emit) {
-  if constexpr (MFMA && sizeof(T) == 2) {
-    tm_f32x4 acc[4];
-    tile_mfma_64(reinterpret_cast<const bf16_t*>(a_row), reinterpret_cast<const bf16_t*>(w_row), K, acc, lds.mfma);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                                        TileFmaLds& lds, Emit emit) {
+  float acc[4][4];
+  tile_fma_64(a_row, w_row, K, acc, lds);
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      const float v[4] = {acc[mt][0], acc[mt][1], acc[mt][2], acc[mt][3]};
-      emit(16 * mt + (lane & 15), 16 * wave + 4 * (lane >> 4), v);
-    }
-  } else {
-    float acc[4][4];
-    tile_fma_64(a_row, w_row, K, acc, lds.fma);
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) emit(ty * 4 + i, tx * 4, acc[i]);
-  }
+  for (int i = 0; i < 4; ++i) emit(ty * 4 + i, tx * 4, acc[i]);
 }
 
 // Whether rows that start at `p` and lie `stride` elements apart (and `stride2` for a second index) can be read
@@ -164,14 +86,20 @@ __host__ __device__ inline bool tile_rows_aligned(const void* p, long stride, lo
   return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && (stride & 7) == 0 && (stride2 & 7) == 0;
 }
 
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 tm_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float tm_f32x4;
+
 // ---- a larger tile on the matrix cores: BM rows of A (128, or 32 for steps of few rows) x 128 rows of W ------------
 // 256 threads = 4 waves, 2 x 2 over the tile at BM = 128 (64 x 64 a wave: 4 x 4 accumulators) and 1 x 4 at BM = 32
 // (32 x 32 a wave).  K is walked in steps of 64 through one LDS stage; the global loads run two steps ahead of the
 // matrix instructions in two sets of registers (the loads of step i + 2 are issued before the matrix instructions
 // of step i and stored to LDS after those of step i + 1), every load unconditional so that a wait for the older
 // set leaves the newer in flight: a row that the tile does not have is read from the tile's first row (its sums
-// are never handed on), and values of k past K are read from the row's end and set to zero by a select.  Operand
-// fragments and the result's layout are those of tile_mfma_64: a lane ends with four consecutive columns of one row.
+// are never handed on), and values of k past K are read from the row's end and set to zero by a select.
+// v_mfma_f32_16x16x32_bf16 with 16 rows of W as its first operand and 16 rows of A as its second: lane
+// (r = lane % 16, q = lane / 16) ends with D[column 4 q + e of W's 16][row r of A's 16], e = 0..3, so a lane holds
+// four consecutive columns of one row of the result, as a thread of the fp32 tile above does.  Every element is
+// summed in an order that depends on K alone.
 // `a_row(r)` / `w_row(r)`: row r of the tile's A / W (16-byte aligned, K a multiple of 8 and at least 8); row 0
 // always exists.
 #define TB_KS 64
