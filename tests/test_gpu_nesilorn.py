@@ -364,3 +364,46 @@ def test_greedy_generation_through_the_scheduler(models):
         for _ in range(12):
             toks.append(int(PN.forward(cfg, w, toks)[-1].argmax()))
         assert list(got) == toks[len(p):], (p, got, toks[len(p):])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_and_generate_programs(models, tmp_path, dtype):
+    """bin/trace_run and bin/generate as a user starts them, on a Nesilorn folder: the model class comes from
+    config.json; steps on standard input, logits in files; generated tokens on standard output."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    d, cfg, w, _, _, reqs, ref = models["N4"]
+    prompt_len = {r: max(2, len(t) - 12) for r, t in reqs.items()}
+    steps, max_tokens = TT.trace_mixed(reqs, prompt_len, seed=4)
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(max_tokens)],
+                          input="".join(json.dumps(s) + "\n" for s in steps), text=True, capture_output=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    pos, got = {}, {}
+    for s in steps:
+        n_want = sum(len(e["want"]) for e in s["entries"])
+        arr = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(n_want, cfg["vocab"])
+        row = 0
+        for e in s["entries"]:
+            base = pos.get(e["id"], 0)
+            for k in e["want"]:
+                got[(e["id"], base + k)] = torch.from_numpy(arr[row].copy())
+                row += 1
+            pos[e["id"]] = base + len(e["tokens"])
+    _check(got, ref, dtype, f"trace_run N4 {dtype} mixed", "N4")
+    if dtype == "float32":
+        prompt = reqs["r4"][:9]
+        gen = subprocess.run([sys.executable, os.path.join(root, "bin", "generate"), "-m", d, "--prompt-ids",
+                              ",".join(map(str, prompt)), "-n", "6", "--greedy", "--dtype", "float32"],
+                             text=True, capture_output=True, timeout=600)
+        assert gen.returncode == 0, gen.stderr[-3000:]
+        toks = list(prompt)
+        for _ in range(6):
+            toks.append(int(PN.forward(cfg, w, toks)[-1].argmax()))
+        assert " " + " ".join(map(str, toks[9:])) + "\n" in gen.stdout, gen.stdout[-2000:]
