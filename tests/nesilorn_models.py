@@ -51,7 +51,7 @@ N3 = {"architecture": "Nesilorn", "vocab": 256, "width": 128, "embedding": {"sca
       ]}
 # N4: no routed layer (nothing hangs on a close call of a router, so bfloat16 is held to its tolerance at every
 #     place); head sizes 80 and 32 for the matrix-core attention kernels; windows at and across page borders.
-N4 = {"architecture": "Nesilorn", "vocab": 300, "width": 96, "embedding": {"scale": 0.5}, "norm": {"eps": 1e-6},
+N4 = {"architecture": "Nesilorn", "vocab": 300, "width": 96, "embedding": {"scale": 0.625}, "norm": {"eps": 2e-6},
       "layers": [
           _layer(_mixer(6, 16, 16, 16, 64, 32), {"kind": "dense", "ff": 160}),
           _layer(_mixer(18, 8, 8, 8, 24, 17, base=3000.0), None),
