@@ -159,17 +159,17 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
   });
 }
 
-// The same on tiles of BM x 128 (tile_mfma_big): grid (tiles of 128 of the 2 ff columns, ceil(P / BM) + E).
-template <int BM>
-__global__ __launch_bounds__(256) void moe_gate_up_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wgu,
+// The same on tiles of BM x BN (tile_mfma_big): grid (tiles of BN of the 2 ff columns, ceil(P / BM) + E).
+template <int BM, int BN>
+__global__ __launch_bounds__(BN == 256 ? 512 : 256) void moe_gate_up_big_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ Wgu,
                                                               bf16_t* __restrict__ y, const int* __restrict__ offsets,
                                                               const int* __restrict__ perm, int E, int top, int W,
                                                               int ff, float limit, float alpha) {
-  __shared__ TileBigLds<BM> lds;
+  __shared__ TileBigLds<BM, BN> lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
-  const int n0 = blockIdx.x * TB_N;
-  tile_mfma_big<BM>(
+  const int n0 = blockIdx.x * BN;
+  tile_mfma_big<BM, BN>(
       [&](int r) { return x + (size_t)(perm[first + r] / top) * W; },
       [&](int r) { return Wgu + ((size_t)e * 2 * ff + n0 + r) * W; }, last - first, 2 * ff - n0, W, lds,
       [&](int i, int j0, const float* v) {
@@ -200,13 +200,14 @@ extern "C" int ia_moe_gate_up(const void* x, const void* Wgu, void* y, const int
                                                                perm, E, top, W, ff, limit, alpha);
   else if (dtype == IA_BF16 && tile_rows_aligned(x, W) && tile_rows_aligned(Wgu, W)) {
     const int bm = moe_tile_rows(P, E);
-    dim3 big((2 * ff + TB_N - 1) / TB_N, (P + bm - 1) / bm + E);
+    const int bn = bm == 128 ? 256 : TB_N;
+    dim3 big((2 * ff + bn - 1) / bn, (P + bm - 1) / bm + E);
     if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
     if (bm == 128)
-      moe_gate_up_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
+      moe_gate_up_big_kernel<128, 256><<<big, 512, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
                                                            perm, E, top, W, ff, limit, alpha);
     else
-      moe_gate_up_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
+      moe_gate_up_big_kernel<32, TB_N><<<big, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)Wgu, (bf16_t*)y, offsets,
                                                           perm, E, top, W, ff, limit, alpha);
   }
   else if (dtype == IA_BF16)
@@ -246,16 +247,16 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ y, 
   });
 }
 
-template <int BM>
-__global__ __launch_bounds__(256) void moe_down_big_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ Wd,
+template <int BM, int BN>
+__global__ __launch_bounds__(BN == 256 ? 512 : 256) void moe_down_big_kernel(const bf16_t* __restrict__ y, const bf16_t* __restrict__ Wd,
                                                            float* __restrict__ parts, const float* __restrict__ weights,
                                                            const int* __restrict__ offsets, const int* __restrict__ perm,
                                                            int E, int top, int N, int W, int ff) {
-  __shared__ TileBigLds<BM> lds;
+  __shared__ TileBigLds<BM, BN> lds;
   int e, first, last;
   if (!moe_tile(offsets, E, blockIdx.y, e, first, last, BM)) return;
-  const int n0 = blockIdx.x * TB_N;
-  tile_mfma_big<BM>(
+  const int n0 = blockIdx.x * BN;
+  tile_mfma_big<BM, BN>(
       [&](int r) { return y + (size_t)(first + r) * ff; },
       [&](int r) { return Wd + ((size_t)e * W + n0 + r) * ff; }, last - first, W - n0, ff, lds,
       [&](int i, int j0, const float* v) {
@@ -285,13 +286,14 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
                                                             perm, E, top, N, W, ff);
   else if (dtype == IA_BF16 && tile_rows_aligned(y, ff) && tile_rows_aligned(Wd, ff)) {
     const int bm = moe_tile_rows(P, E);
-    dim3 big((W + TB_N - 1) / TB_N, (P + bm - 1) / bm + E);
+    const int bn = bm == 128 ? 256 : TB_N;
+    dim3 big((W + bn - 1) / bn, (P + bm - 1) / bm + E);
     if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
     if (bm == 128)
-      moe_down_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
+      moe_down_big_kernel<128, 256><<<big, 512, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
                                                         perm, E, top, N, W, ff);
     else
-      moe_down_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
+      moe_down_big_kernel<32, TB_N><<<big, 256, 0, stream>>>((const bf16_t*)y, (const bf16_t*)Wd, parts, weights, offsets,
                                                        perm, E, top, N, W, ff);
   }
   else if (dtype == IA_BF16)

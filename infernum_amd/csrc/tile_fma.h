@@ -106,29 +106,36 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float tm_f32x4;
 #define TB_LD 72
 #define TB_N 128
 
-template <int BM>
+// BN = 256 (with BM = 128): eight waves, 2 x 4 over the tile, for products of many rows: the rows of A are read
+// once for twice the columns (85 flops a byte read into LDS where 128 x 128 has 64).
+template <int BM, int BN = TB_N>
 struct TileBigLds {
   uint16_t a[BM][TB_LD];
-  uint16_t w[TB_N][TB_LD];
+  uint16_t w[BN][TB_LD];
 };
 
-template <int BM, typename ARow, typename WRow, typename Emit>
+template <int BM, int BN>
+constexpr int tile_big_threads() { return BN == 256 ? 512 : 256; }
+
+template <int BM, int BN = TB_N, typename ARow, typename WRow, typename Emit>
 __device__ __forceinline__ void tile_mfma_big(ARow a_row, WRow w_row, int a_rows, int w_rows, int K,
-                                              TileBigLds<BM>& lds, Emit emit) {
-  static_assert(BM == 128 || BM == 32, "tiles of 128 or 32 rows");
-  constexpr int WM = BM == 128 ? 2 : 1, WN = 4 / WM;           // waves along the rows and the columns
-  constexpr int MT = BM / WM / 16, NT = TB_N / WN / 16;       // 16 x 16 tiles a wave
-  constexpr int AR = BM / 32, WR = TB_N / 32;                 // rows of A and of W that a thread loads a step
+                                              TileBigLds<BM, BN>& lds, Emit emit) {
+  static_assert((BM == 128 || BM == 32) && (BN == 128 || (BN == 256 && BM == 128)), "tiles of 128 x 128, 32 x 128, 128 x 256");
+  constexpr int WAVES = tile_big_threads<BM, BN>() / 64;
+  constexpr int WM = BM == 128 ? 2 : 1, WN = WAVES / WM;       // waves along the rows and the columns
+  constexpr int MT = BM / WM / 16, NT = BN / WN / 16;         // 16 x 16 tiles a wave
+  constexpr int RP = WAVES * 8;                               // rows that the workgroup's threads read in one pass
+  constexpr int AR = BM / RP, WR = BN / RP;                   // rows of A and of W that a thread loads a step
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, q = lane >> 4;
-  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (TB_N / WN);
+  const int wm0 = (wave / WN) * (BM / WM), wn0 = (wave % WN) * (BN / WN);
   const int lr = tid >> 3, lk = (tid & 7) * 8;                // 8 threads read a row's 64 values of k
   const bf16_t* ap[AR];
   const bf16_t* wp[WR];
 #pragma unroll
-  for (int s = 0; s < AR; ++s) ap[s] = a_row(lr + 32 * s < a_rows ? lr + 32 * s : 0);
+  for (int s = 0; s < AR; ++s) ap[s] = a_row(lr + RP * s < a_rows ? lr + RP * s : 0);
 #pragma unroll
-  for (int s = 0; s < WR; ++s) wp[s] = w_row(lr + 32 * s < w_rows ? lr + 32 * s : 0);
+  for (int s = 0; s < WR; ++s) wp[s] = w_row(lr + RP * s < w_rows ? lr + RP * s : 0);
   tm_f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -152,9 +159,9 @@ __device__ __forceinline__ void tile_mfma_big(ARow a_row, WRow w_row, int a_rows
   };
   auto stage = [&](const uint4 (&xa)[AR], const uint4 (&xw)[WR]) {
 #pragma unroll
-    for (int s = 0; s < AR; ++s) *reinterpret_cast<uint4*>(&lds.a[lr + 32 * s][lk]) = xa[s];
+    for (int s = 0; s < AR; ++s) *reinterpret_cast<uint4*>(&lds.a[lr + RP * s][lk]) = xa[s];
 #pragma unroll
-    for (int s = 0; s < WR; ++s) *reinterpret_cast<uint4*>(&lds.w[lr + 32 * s][lk]) = xw[s];
+    for (int s = 0; s < WR; ++s) *reinterpret_cast<uint4*>(&lds.w[lr + RP * s][lk]) = xw[s];
   };
   auto multiply = [&]() {
 #pragma unroll
