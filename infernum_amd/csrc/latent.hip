@@ -96,7 +96,8 @@ __global__ __launch_bounds__(256) void gemm_heads_kernel(const T* __restrict__ x
   });
 }
 
-// The same on tiles of BM x 128 (tile_mfma_big): grid (tiles of 128 of Nout, tiles of BM of N, H).
+// The same on tiles of BM x 128 (tile_mfma_big): grid (tiles of 128 of Nout, tiles of BM of N, H).  With 2,048 rows
+// tiles of 32 rows took 18 and 26 us where tiles of 128 took 30 and 28 (heads of 224 x 64 and 64 x 224).
 template <int BM>
 __global__ __launch_bounds__(256) void gemm_heads_big_kernel(const bf16_t* __restrict__ x, int x_row, int x_head,
                                                              const bf16_t* __restrict__ W, bf16_t* __restrict__ out,
@@ -139,16 +140,12 @@ extern "C" int ia_gemm_heads(const void* x, int x_row, int x_head, const void* W
                                                               (float*)out, o_row, o_head, (const float*)gate, g_row,
                                                               N, Nout, K);
   else if (dtype == IA_BF16 && (K & 7) == 0 && tile_rows_aligned(x, x_row, x_head) && tile_rows_aligned(W, K)) {
-    const int bm = N >= 96 ? 128 : 32;
+    const int bm = 32;      // K is short here (a head's size): many small workgroups hide each other's few steps better than few large ones
     dim3 big((Nout + TB_N - 1) / TB_N, (N + bm - 1) / bm, H);
-    if (bm == 128)
-      gemm_heads_big_kernel<128><<<big, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
-                                                          (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
-                                                          Nout, K);
-    else
-      gemm_heads_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
-                                                         (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
-                                                         Nout, K);
+    if (big.y > 65535u) return IA_ERR_UNSUPPORTED;
+    gemm_heads_big_kernel<32><<<big, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
+                                                       (bf16_t*)out, o_row, o_head, (const bf16_t*)gate, g_row, N,
+                                                       Nout, K);
   }
   else if (dtype == IA_BF16)
     gemm_heads_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)W,
