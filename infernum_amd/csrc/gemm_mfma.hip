@@ -38,13 +38,19 @@ typedef const __attribute__((address_space(1))) void* gm_global_ptr;
 typedef __attribute__((address_space(3))) void* gm_lds_ptr;
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int FILL_STEPS, bool SPLIT, bool GLU = false,
-          bool WT = false>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X,
-                                                                           const uint16_t* __restrict__ W,
-                                                                           uint16_t* __restrict__ C,
-                                                                           float* __restrict__ P, int M, int N,
+          bool WT = false, bool GROUPED = false>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const uint16_t* __restrict__ X_all,
+                                                                           const uint16_t* __restrict__ W_all,
+                                                                           uint16_t* __restrict__ C_all,
+                                                                           float* __restrict__ P, int M_all, int N,
                                                                            int K, int tiles_m, int tiles_n,
-                                                                           int splits) {
+                                                                           int splits,
+                                                                           const int* __restrict__ group_rows_at = nullptr,
+                                                                           int groups = 0) {
+  const uint16_t* X = X_all;
+  const uint16_t* W = W_all;
+  uint16_t* C = C_all;
+  int M = M_all;
   constexpr int WAVES = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // tile of a wave
   constexpr int TM = WM / 32, TN = WN / 32;             // in accumulator tiles of 32 x 32
@@ -59,9 +65,17 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
 
   // workgroups go to the 8 dies in turn (workgroup i to die i % 8), and each die has an L2 of its own:
   // give every die one contiguous run of tiles, so that W is read from memory once and not once per die
-  const int tiles = tiles_m * tiles_n;
+  int tiles_m_here = tiles_m;
+  if constexpr (GROUPED) {
+    // the tiles of rows that the groups have in this step (the launch has one for every case): the dies share
+    // those evenly, and the workgroups beyond them leave
+    tiles_m_here = 0;
+    for (int g = 0; g < groups; ++g) tiles_m_here += (group_rows_at[g + 1] - group_rows_at[g] + BM - 1) / BM;
+  }
+  const int tiles = tiles_m_here * tiles_n;
   const int total = SPLIT ? tiles * splits : tiles;
   const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  if (GROUPED && idx >= (total >> 3) + (xcd < (total & 7) ? 1 : 0)) return;
   int bid = xcd * (total >> 3) + min(xcd, total & 7) + idx;
   // with K split over workgroups, part p of every tile comes before part p + 1 of any: the tiles of M under one
   // tile of N still run side by side on one die
@@ -71,10 +85,35 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_mfma_kernel(const
   const int GROUP = 8;
   const int per_group = GROUP * tiles_n;
   const int group = bid / per_group, in_group = bid - group * per_group;
-  const int group_rows = min(GROUP, tiles_m - group * GROUP);
+  const int group_rows = min(GROUP, tiles_m_here - group * GROUP);
   const int tm = group * GROUP + in_group % group_rows;
   const int tn = in_group / group_rows;
-  const int m0 = tm * BM, n0 = tn * BN;
+  int m0 = tm * BM;
+  const int n0 = tn * BN;
+  if constexpr (GROUPED) {
+    // GROUPED: rows group_rows_at[g] .. group_rows_at[g + 1] - 1 of X are multiplied with matrix g of W [groups, N, K],
+    // and tm counts tiles of BM rows over the groups one after the other (a group's last tile is filled in part; the
+    // launch has a tile for every case and the spare workgroups leave here): from here on the workgroup sees its
+    // group's rows from the tile's first on as the whole of X and C.
+    static_assert(!GROUPED || (!SPLIT && !GLU && !WT), "the grouped product leaves whole bf16 sums");
+    int seen = 0, g = 0, first = 0, last = 0;
+    for (; g < groups; ++g) {
+      const int lo = group_rows_at[g], hi = group_rows_at[g + 1];
+      const int t = (hi - lo + BM - 1) / BM;
+      if (tm < seen + t) {
+        first = lo + (tm - seen) * BM;
+        last = hi;
+        break;
+      }
+      seen += t;
+    }
+    if (g >= groups) return;
+    X += (size_t)first * K;
+    C += (size_t)first * N;
+    W += (size_t)g * N * K;
+    M = last - first;
+    m0 = 0;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -443,8 +482,34 @@ extern "C" int ia_gemm_mfma_swiglu(const void* X, const void* W, int w_tiled, vo
                                                              nullptr, M, N, K, 1, stream);
 }
 
+// Grouped: rows rows_at[g] .. rows_at[g + 1] - 1 of X [rows, K] times matrix g of W [groups, N, K], into the same rows
+// of C [rows, N]; rows_at [groups + 1] lies on the device (nothing is read back: the launch has a tile for every way
+// the rows can fall into groups).  Tiles of 128 x 256, three stages.
+extern "C" int ia_gemm_mfma_grouped(const void* X, const void* W, void* C, const int* rows_at, int groups, int rows,
+                                    int N, int K, hipStream_t stream) {
+  if (groups <= 0 || !rows_at) return IA_ERR_BAD_ARG;
+  if (rows == 0) return IA_OK;
+  if (!gemm_mfma_takes(rows, N, K)) return IA_ERR_UNSUPPORTED;
+  constexpr int BM = 128, BN = 256, STAGES = 3;
+  const int tiles_m = (rows + BM - 1) / BM + groups, tiles_n = (N + BN - 1) / BN;
+  const size_t lds_bytes = (size_t)STAGES * (BM + BN) * GM_ROW_BYTES;
+  auto kernel = gemm_mfma_kernel<BM, BN, 2, 2, STAGES, 2, false, false, false, true>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    configured = true;
+  }
+  if ((long long)tiles_m * tiles_n > 0x7fffffffLL) return IA_ERR_UNSUPPORTED;
+  kernel<<<tiles_m * tiles_n, 256, lds_bytes, stream>>>((const uint16_t*)X, (const uint16_t*)W, (uint16_t*)C, nullptr,
+                                                        rows, N, K, tiles_m, tiles_n, 1, rows_at, groups);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 // ---- the launchers of this file as operations of a step's program (see op_call.h) ----
 #include "op_call.h"
 IA_OP(ia_gemm_mfma)
 IA_OP(ia_gemm_mfma_split)
 IA_OP(ia_gemm_mfma_swiglu)
+IA_OP(ia_gemm_mfma_grouped)

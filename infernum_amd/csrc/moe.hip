@@ -305,8 +305,94 @@ extern "C" int ia_moe_down(const void* y, const void* Wd, float* parts, const fl
   return IA_OK;
 }
 
+// ---- the experts of a step of many rows by the grouped form of the LDS-tiled product (ia_gemm_mfma_grouped) ----------
+// The tokens' rows are first brought into the order of the sort (an expert's rows one after the other), the two
+// products run expert by expert over those rows, and the activation and the routing weight are passes of their own:
+//   ia_moe_gather   xs[p, :] = x[perm[p] / top, :]
+//   ia_moe_glu      y[p, j] = g sigmoid(alpha g) (u + 1), g = min(gu[p, 2 j], limit), u = clamp(gu[p, 2 j + 1], +-limit)
+//   ia_moe_scatter  parts[choice, token, :] = float(o[p, :]) * weights[perm[p]]
+// All three in bfloat16 with rows that are read 16 bytes at a time.
+__global__ __launch_bounds__(256) void moe_gather_kernel(const uint4* __restrict__ x, const int* __restrict__ perm,
+                                                         uint4* __restrict__ xs, int top, int pieces) {
+  const int p = blockIdx.x;
+  const uint4* src = x + (size_t)(perm[p] / top) * pieces;
+  uint4* dst = xs + (size_t)p * pieces;
+  for (int i = threadIdx.x; i < pieces; i += 256) dst[i] = src[i];
+}
+
+extern "C" int ia_moe_gather(const void* x, const int* perm, void* xs, int P, int top, int W, hipStream_t stream) {
+  if (P < 0 || top <= 0 || W <= 0) return IA_ERR_BAD_ARG;
+  if ((W & 7) || ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(xs)) & 15)) return IA_ERR_UNSUPPORTED;
+  if (P == 0) return IA_OK;
+  moe_gather_kernel<<<P, 256, 0, stream>>>((const uint4*)x, perm, (uint4*)xs, top, W / 8);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+__global__ __launch_bounds__(256) void moe_glu_kernel(const uint4* __restrict__ gu, uint2* __restrict__ y, size_t n4,
+                                                      float limit, float alpha) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+    const uint4 v = gu[i];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float g = fminf(__uint_as_float(w[k] << 16), limit);
+      const float u = fminf(fmaxf(__uint_as_float(w[k] & 0xffff0000u), -limit), limit);
+      o[k] = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f);
+    }
+    uint2 r;
+    r.x = (uint32_t)float_to_bf16_bits(o[0]) | ((uint32_t)float_to_bf16_bits(o[1]) << 16);
+    r.y = (uint32_t)float_to_bf16_bits(o[2]) | ((uint32_t)float_to_bf16_bits(o[3]) << 16);
+    y[i] = r;
+  }
+}
+
+extern "C" int ia_moe_glu(const void* gu, void* y, int P, int ff, float limit, float alpha, hipStream_t stream) {
+  if (P < 0 || ff <= 0) return IA_ERR_BAD_ARG;
+  if ((ff & 3) || ((reinterpret_cast<uintptr_t>(gu) | reinterpret_cast<uintptr_t>(y)) & 15)) return IA_ERR_UNSUPPORTED;
+  const size_t n4 = (size_t)P * ff / 4;
+  if (n4 == 0) return IA_OK;
+  const unsigned grid = (unsigned)((n4 + 255) / 256 < 65536 ? (n4 + 255) / 256 : 65536);
+  moe_glu_kernel<<<grid, 256, 0, stream>>>((const uint4*)gu, (uint2*)y, n4, limit, alpha);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const uint4* __restrict__ o, const int* __restrict__ perm,
+                                                          const float* __restrict__ weights, float* __restrict__ parts,
+                                                          int N, int top, int W) {
+  const int p = blockIdx.x;
+  const int pair = perm[p];
+  const int token = pair / top, choice = pair - token * top;
+  const float wt = weights[pair];
+  const uint4* src = o + (size_t)p * (W / 8);
+  float4* dst = reinterpret_cast<float4*>(parts + ((size_t)choice * N + token) * W);
+  for (int i = threadIdx.x; i < W / 8; i += 256) {
+    const uint4 v = src[i];
+    dst[2 * i] = make_float4(__uint_as_float(v.x << 16) * wt, __uint_as_float(v.x & 0xffff0000u) * wt,
+                             __uint_as_float(v.y << 16) * wt, __uint_as_float(v.y & 0xffff0000u) * wt);
+    dst[2 * i + 1] = make_float4(__uint_as_float(v.z << 16) * wt, __uint_as_float(v.z & 0xffff0000u) * wt,
+                                 __uint_as_float(v.w << 16) * wt, __uint_as_float(v.w & 0xffff0000u) * wt);
+  }
+}
+
+extern "C" int ia_moe_scatter(const void* o, const int* perm, const float* weights, float* parts, int N, int top,
+                              int W, hipStream_t stream) {
+  if (N < 0 || top <= 0 || W <= 0) return IA_ERR_BAD_ARG;
+  if ((W & 7) || ((reinterpret_cast<uintptr_t>(o) | reinterpret_cast<uintptr_t>(parts)) & 15)) return IA_ERR_UNSUPPORTED;
+  if (N == 0) return IA_OK;
+  moe_scatter_kernel<<<N * top, 256, 0, stream>>>((const uint4*)o, perm, weights, parts, N, top, W);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 #include "op_call.h"
 IA_OP(ia_router_topk)
 IA_OP(ia_moe_sort)
 IA_OP(ia_moe_gate_up)
 IA_OP(ia_moe_down)
+IA_OP(ia_moe_gather)
+IA_OP(ia_moe_glu)
+IA_OP(ia_moe_scatter)

@@ -289,6 +289,23 @@ def router_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
     return ids, weights
 
 
+MOE_GROUPED_ROWS_AN_EXPERT = 48
+
+
+def moe_grouped_from_tokens(E: int, top: int, W: int, ff: int, dtype: torch.dtype) -> int:
+    """From how many tokens of a step on the routed experts take the grouped form of the LDS-tiled product (an
+    expert then has some tens of rows on average); 0: never (32-bit, or sizes that product does not take: its
+    inner dimensions W and ff must be multiples of 64)."""
+    if dtype != torch.bfloat16 or W % 64 or ff % 64:
+        return 0
+    return -(-MOE_GROUPED_ROWS_AN_EXPERT * E // top)
+
+
+def moe_grouped_rows(N: int, E: int, top: int, W: int, ff: int, dtype: torch.dtype) -> bool:
+    first = moe_grouped_from_tokens(E, top, W, ff, dtype)
+    return first > 0 and N >= first
+
+
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
                 w_down: torch.Tensor, limit: float, alpha: float) -> SplitSum:
     """The chosen experts of every token: w_gate_up [E, 2 ff, W] with the gate's and up's rows alternating,
@@ -310,6 +327,18 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     parts = torch.empty((top, N, W), dtype=torch.float32, device=x.device)
     code = DTYPE_CODE[x.dtype]
     _ok(_core().ia_moe_sort(_p(ids), _p(offsets), _p(perm), P, E, _stream()), "moe_sort")
+    if moe_grouped_rows(N, E, top, W, ff, x.dtype):
+        # many rows an expert: the tokens' rows in the order of the sort, the LDS-tiled product expert by expert
+        xs = torch.empty((P, W), dtype=x.dtype, device=x.device)
+        gu = torch.empty((P, 2 * ff), dtype=x.dtype, device=x.device)
+        _ok(_core().ia_moe_gather(_p(x), _p(perm), _p(xs), P, top, W, _stream()), "moe_gather")
+        _ok(_core().ia_gemm_mfma_grouped(_p(xs), _p(w_gate_up), _p(gu), _p(offsets), E, P, 2 * ff, W, _stream()),
+            "gemm_mfma_grouped")
+        _ok(_core().ia_moe_glu(_p(gu), _p(y), P, ff, ctypes.c_float(limit), ctypes.c_float(alpha), _stream()), "moe_glu")
+        _ok(_core().ia_gemm_mfma_grouped(_p(y), _p(w_down), _p(xs), _p(offsets), E, P, W, ff, _stream()),
+            "gemm_mfma_grouped")
+        _ok(_core().ia_moe_scatter(_p(xs), _p(perm), _p(weights), _p(parts), N, top, W, _stream()), "moe_scatter")
+        return SplitSum(parts)
     _ok(_core().ia_moe_gate_up(_p(x), _p(w_gate_up), _p(y), _p(offsets), _p(perm), code, P, E, top, W, ff,
                                ctypes.c_float(limit), ctypes.c_float(alpha), _stream()), "moe_gate_up")
     _ok(_core().ia_moe_down(_p(y), _p(w_down), _p(parts), _p(weights), _p(offsets), _p(perm), code, N, E, top, W, ff,

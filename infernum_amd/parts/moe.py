@@ -92,10 +92,24 @@ class RoutedExperts(FeedForward):
         program.op("core", "ia_router_topk", [z.tensor(), b, K.DTYPE_CODE[b.dtype] if b is not None else 0, ids, wts,
                                               N, E, top, STREAM])
         program.op("core", "ia_moe_sort", [ids, offsets, perm, N * top, E, STREAM])
+        from ..engine.program import NEVER, Guard
+        first = K.moe_grouped_from_tokens(E, top, H, I, self.rt.dtype)
+        grouped = Guard.between(N, first) if first > 0 else NEVER
+        tiled = ~grouped
         program.op("core", "ia_moe_gate_up", [program.x, self.w_gate_up, y, offsets, perm, program.act_code, N * top,
-                                              E, top, H, I, self.limit, self.alpha, STREAM])
+                                              E, top, H, I, self.limit, self.alpha, STREAM], tiled)
         program.op("core", "ia_moe_down", [y, self.w_down, parts, wts, offsets, perm, program.act_code, N, E, top, H,
-                                           I, STREAM])
+                                           I, STREAM], tiled)
+        if first > 0 and first <= T:
+            # steps of many tokens: the grouped form of the LDS-tiled product (kernels.api.moe_experts)
+            xs = program.buffer("moe.sorted", T * top * H * program.act_bytes)
+            gu = program.buffer("moe.gate_up", T * top * 2 * I * program.act_bytes)
+            program.op("core", "ia_moe_gather", [program.x, perm, xs, N * top, top, H, STREAM], grouped)
+            program.op("core", "ia_gemm_mfma_grouped", [xs, self.w_gate_up, gu, offsets, E, N * top, 2 * I, H, STREAM],
+                       grouped)
+            program.op("core", "ia_moe_glu", [gu, y, N * top, I, self.limit, self.alpha, STREAM], grouped)
+            program.op("core", "ia_gemm_mfma_grouped", [y, self.w_down, xs, offsets, E, N * top, H, I, STREAM], grouped)
+            program.op("core", "ia_moe_scatter", [xs, perm, wts, parts, N, top, H, STREAM], grouped)
         program.pending = Value(H, [Alt(ALWAYS, parts, top, torch.float32)])
 
 

@@ -7,7 +7,8 @@ N2: sizes that no fast kernel takes (latent head size 26, width 100, odd vocabul
     two experts; a window of one token (a query sees itself alone) and a layer without a mask; a scale of 1.
 N4: see below.
 N3: twenty heads on the one cached head (more than one tile of sixteen heads); plain query size equal to the
-    latent's; rotated part partly rotated (rot.dims below rot_dim); eight experts, three chosen.
+    latent's; rotated part partly rotated (rot.dims below rot_dim); four experts, three chosen, of sizes that
+    send portions of 64 tokens and more to the grouped product and shorter ones to the tiles.
 """
 import json
 import os
@@ -46,7 +47,7 @@ N2 = {"architecture": "Nesilorn", "vocab": 333, "width": 100, "embedding": {"sca
       ]}
 N3 = {"architecture": "Nesilorn", "vocab": 256, "width": 128, "embedding": {"scale": 2.5}, "norm": {"eps": 3e-6},
       "layers": [
-          _layer(_mixer(20, 64, 32, 16, 64, 48, base=1000000.0, dims=16), _moe(32, 8, 3, 2.0)),
+          _layer(_mixer(20, 64, 32, 16, 64, 48, base=1000000.0, dims=16), _moe(64, 4, 3, 2.0)),
           _layer(_mixer(20, 64, 32, 16, 64, 48, base=1000000.0, dims=16), {"kind": "dense", "ff": 200}),
       ]}
 # N4: no routed layer (nothing hangs on a close call of a router, so bfloat16 is held to its tolerance at every

@@ -109,7 +109,8 @@ def test_router_choice_and_weights(E, top, n):
 
 @BOTH
 @pytest.mark.parametrize("H,I,E,top,limit,n", [(64, 24, 5, 2, 1.5, 40), (100, 20, 3, 1, 0.5, 9), (96, 36, 2, 2, 3.0, 70),
-                                               (128, 64, 16, 4, 2.0, 260), (64, 16, 8, 3, 1.0, 1)])
+                                               (128, 64, 16, 4, 2.0, 260), (64, 16, 8, 3, 1.0, 1),
+                                               (192, 128, 4, 2, 1.5, 300), (192, 128, 4, 2, 1.5, 95)])
 def test_routed_experts(dtype, H, I, E, top, limit, n):
     """Against the plain experts, with inputs large enough that the limit cuts gate and up values on both sides;
     a router whose bias alone decides (weights zero) shows the bias; every expert gets tokens, some none."""
