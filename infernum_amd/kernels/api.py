@@ -289,6 +289,23 @@ def router_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
     return ids, weights
 
 
+def gemm_mfma_grouped(x: torch.Tensor, w: torch.Tensor, rows_at: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[rows_at[g] : rows_at[g + 1]] = x[rows_at[g] : rows_at[g + 1]] @ w[g]^T for every group g: x [rows, K] and
+    w [groups, N, K] in bf16, rows_at int32 [groups + 1] on the device, rising from 0 to at most rows (nothing of it
+    is read on the host; rows past rows_at[-1] are left as they are).  K must be a multiple of 64."""
+    _dev(x, w, rows_at, out)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 3
+          and w.shape[2] == x.shape[1], "gemm_mfma_grouped: x [rows, K] and w [groups, N, K] in bf16")
+    G, N, Kd = w.shape
+    _i32(rows_at, G + 1, "gemm_mfma_grouped rows_at")
+    if out is None:
+        out = torch.empty((x.shape[0], N), dtype=torch.bfloat16, device=x.device)
+    _need(out.dtype == torch.bfloat16 and tuple(out.shape) == (x.shape[0], N), "gemm_mfma_grouped: out [rows, N] in bf16")
+    _ok(_core().ia_gemm_mfma_grouped(_p(x), _p(w), _p(out), _p(rows_at), G, x.shape[0], N, Kd, _stream()),
+        "gemm_mfma_grouped")
+    return out
+
+
 MOE_GROUPED_ROWS_AN_EXPERT = 48
 
 
@@ -332,11 +349,9 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
         xs = torch.empty((P, W), dtype=x.dtype, device=x.device)
         gu = torch.empty((P, 2 * ff), dtype=x.dtype, device=x.device)
         _ok(_core().ia_moe_gather(_p(x), _p(perm), _p(xs), P, top, W, _stream()), "moe_gather")
-        _ok(_core().ia_gemm_mfma_grouped(_p(xs), _p(w_gate_up), _p(gu), _p(offsets), E, P, 2 * ff, W, _stream()),
-            "gemm_mfma_grouped")
+        gemm_mfma_grouped(xs, w_gate_up, offsets, gu)
         _ok(_core().ia_moe_glu(_p(gu), _p(y), P, ff, ctypes.c_float(limit), ctypes.c_float(alpha), _stream()), "moe_glu")
-        _ok(_core().ia_gemm_mfma_grouped(_p(y), _p(w_down), _p(xs), _p(offsets), E, P, W, ff, _stream()),
-            "gemm_mfma_grouped")
+        gemm_mfma_grouped(y, w_down, offsets, xs)
         _ok(_core().ia_moe_scatter(_p(xs), _p(perm), _p(weights), _p(parts), N, top, W, _stream()), "moe_scatter")
         return SplitSum(parts)
     _ok(_core().ia_moe_gate_up(_p(x), _p(w_gate_up), _p(y), _p(offsets), _p(perm), code, P, E, top, W, ff,
@@ -973,7 +988,7 @@ def attention_mfma_available(d: int) -> bool:
 # standard error when the process ends (``profile_report`` gives it at any time).  The reference's switch of the
 # same name prints the time per operation of its graph executor (infernum-cpu/src/executor.rs:24-71).  Steps
 # are not recorded into HIP graphs meanwhile (a replayed launch has no call to bracket).
-_PROFILED = ("norm_add", "activation", "latent_prepare", "gemm_heads", "router_topk", "moe_experts", "cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
+_PROFILED = ("gemm_mfma_grouped", "norm_add", "activation", "latent_prepare", "gemm_heads", "router_topk", "moe_experts", "cast", "copy_pages", "gather_tokens", "words_from_host", "words_to_host", "embed", "add_rmsnorm", "residual_add", "rope_kv_append", "swiglu", "gemm_generic", "gemm_mfma",
              "gemm_library", "gemm_skinny", "gemm_skinny_rows", "attention_generic", "attention_decode", "attention_decode_rotating",
              "attention_prefill", "argmax", "repetition_penalty", "sample")
 _profile_on = False

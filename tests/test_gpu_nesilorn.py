@@ -133,6 +133,26 @@ def test_routed_experts(dtype, H, I, E, top, limit, n):
     assert (g_all > limit).any() and (g_all.abs() < limit).any()
 
 
+@pytest.mark.parametrize("counts,N,Kd", [((0, 1, 128, 129, 0, 300, 7), 200, 128), ((5,), 256, 64), ((130, 0, 0, 126), 520, 192)])
+def test_grouped_product(counts, N, Kd):
+    """Rows in groups of unequal size (empty ones, one row, a tile's 128 and one more), each group with a matrix of
+    its own; rows behind the last group stay as they were."""
+    from infernum_amd.kernels import api as K
+    g = torch.Generator().manual_seed(len(counts) + N)
+    rows = sum(counts) + 3
+    x = (torch.randn(rows, Kd, generator=g)).to(torch.bfloat16)
+    w = (torch.randn(len(counts), N, Kd, generator=g) / Kd ** 0.5).to(torch.bfloat16)
+    at = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32)
+    out = torch.full((rows, N), 7.0, dtype=torch.bfloat16, device=DEV)
+    K.gemm_mfma_grouped(x.to(DEV), w.to(DEV), at.to(DEV), out)
+    for i, n in enumerate(counts):
+        lo = int(at[i])
+        want = x[lo:lo + n].double() @ w[i].double().t()
+        if n:
+            assert rel_err(out[lo:lo + n], want) <= PART_TOL["bfloat16"], i
+    assert torch.equal(out[sum(counts):].cpu(), torch.full((3, N), 7.0, dtype=torch.bfloat16))
+
+
 def _mixer_params(m, W, eps):
     pos = {"kind": "rope", "params": {"head_dim": m["rot_dim"] + m["kv_rank"], "theta": m["rot"]["base"],
                                       "rotary_dim": m["rot"]["dims"]}}
