@@ -31,7 +31,7 @@ from ..parts.base import CacheSpec, CacheView, StateSpec
 from . import native
 from .pages import NO_PAGE, BlockTable, PageAllocator, PageError, pages_for  # noqa: F401  (NO_PAGE: part of this module's face)
 
-_KINDS = {"full": 0, "window": 1}
+_KINDS = {"full": 0, "window": 1, "chunk": 2}
 
 
 class CacheGroup:

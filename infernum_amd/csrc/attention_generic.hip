@@ -7,7 +7,8 @@
 //
 // Key pages are [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d,
 // page_size]; block_tables[s, j / page_size] is the page of key j of sequence s.  The query of token n stands at positions[n] and
-// sees keys max(0, pos - window + 1) .. pos  (window <= 0: all keys from 0).
+// sees keys max(0, pos - window + 1) .. pos  (window 0: all keys from 0; window < 0: the keys of its own
+// chunk of -window positions, see ia_first_visible_key).
 #include "common.h"
 
 #define AG_MAX_D 640
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const T* __restrict__ 
   __syncthreads();
 
   const int j_hi = pos;
-  const int j_lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int j_lo = ia_first_visible_key(pos, window);
   float m = -INFINITY, l = 0.f;
   float acc[AG_MAX_D / 64];
 #pragma unroll

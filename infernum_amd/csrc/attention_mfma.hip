@@ -276,7 +276,7 @@ __global__ __launch_bounds__(WAVES * 64, ((WAVES == 4 && HD <= 128) ? 3 : 1)) vo
   const int* bt = block_tables + (size_t)b * bt_stride;
   const int bt_ahead = tid < bt_stride ? bt[tid] : -1;
   const int p = positions[b];
-  const int lo0 = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo0 = ia_first_visible_key(p, window);
   const int t_first = lo0 / 16, t_last = p / 16;
   const int per = (t_last - t_first + 1 + num_splits - 1) / num_splits;
   const int ta = t_first + split * per;
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
     const int hj = (hc * HGW + hgw) * CT + c;
     const bool ok = hj < G && row < qlen && wave_live;
     pos[c] = ok ? ctx + row : -1;
-    lo[c] = (window > 0 && pos[c] - window + 1 > 0) ? pos[c] - window + 1 : 0;
+    lo[c] = ia_first_visible_key(pos[c], window);
     const uint16_t* qrow = q + (size_t)(qstart + (ok ? row : first_row)) * q_row_stride + (size_t)(g * G + (ok ? hj : 0)) * HD;
 #pragma unroll
     for (int st = 0; st < NS32; ++st) {
@@ -612,10 +612,10 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
 
   // ---- keys the workgroup needs: those its rows may see
   const int key_hi = ctx + last_row;
-  const int key_lo = (window > 0 && ctx + first_row - window + 1 > 0) ? ctx + first_row - window + 1 : 0;
+  const int key_lo = ia_first_visible_key(ctx + first_row, window);
   const int wave_hi = ctx + rb + 15;                                    // last key any row of this wave sees
-  const int wave_lo = (window > 0 && ctx + rb - window + 1 > 0) ? ctx + rb - window + 1 : 0;
-  const int wave_lo_last = (window > 0 && ctx + rb + 15 - window + 1 > 0) ? ctx + rb + 15 - window + 1 : 0;
+  const int wave_lo = ia_first_visible_key(ctx + rb, window);
+  const int wave_lo_last = ia_first_visible_key(ctx + rb + 15, window);
   const int* bt = block_tables + (size_t)sidx * bt_stride;
   const int t_begin = key_lo / PF_KT, t_end = key_hi / PF_KT;          // inclusive
 
@@ -774,7 +774,7 @@ __global__ __launch_bounds__(4 * HGW * 64) void attn_prefill_kernel(
       }
       // ---- softmax statistics per column; probabilities as the B operand of the second product.
       // Only tiles that touch the diagonal or a window's lower edge need the mask (the same for the whole wave).
-      const bool need_mask = (t0 + 31 > ctx + rb) || (window > 0 && t0 < wave_lo_last) || rb + 15 >= qlen;
+      const bool need_mask = (t0 + 31 > ctx + rb) || (window != 0 && t0 < wave_lo_last) || rb + 15 >= qlen;
       bf16x8_t pb[CT];
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
@@ -988,7 +988,7 @@ extern "C" int ia_attn_prefill(const void* q, int q_row_stride, const void* k_pa
   if (launch_shape < 0 || (launch_shape & ~(0xff | IA_PREFILL_PAIRED))) return IA_ERR_BAD_ARG;
   // under a window the rows of the two ends share no keys, and the keys between them may have no page any more:
   // rows are not paired then, whatever was asked for
-  const int heads_per_workgroup = launch_shape & 0xff, paired = ((launch_shape & IA_PREFILL_PAIRED) && window <= 0) ? 1 : 0;
+  const int heads_per_workgroup = launch_shape & 0xff, paired = ((launch_shape & IA_PREFILL_PAIRED) && window == 0) ? 1 : 0;
   if (num_tiles < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || ps <= 0 || (ps & 3) || num_pages <= 0 ||
       bt_stride <= 0 || !(scale > 0.f))
     return IA_ERR_BAD_ARG;

@@ -45,6 +45,7 @@ CORE_SOURCES = [
     "activations.hip",
     "latent.hip",
     "moe.hip",
+    "seqmix.hip",
     "sampling.hip",
     "peaks.hip",
 ]

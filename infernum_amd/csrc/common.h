@@ -123,6 +123,15 @@ __device__ __forceinline__ void rope_pair(float a, float b, float cs, float sn, 
   hi = __builtin_fmaf(a, sn, b * cs);
 }
 
+// The first key that a query at position p sees, from the mask's code: 0 all keys from 0; w > 0 a sliding
+// window, the last w keys (p - w + 1 .. p); w < 0 chunks of -w positions counted from the request's start,
+// the keys of the query's own chunk (floor(p / c) c .. p).  Never decreases with p.
+__host__ __device__ __forceinline__ int ia_first_visible_key(int p, int window) {
+  if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;
+  if (window < 0) return p < 0 ? 0 : p / (-window) * (-window);
+  return 0;
+}
+
 #define IA_LAUNCH_CHECK()                          \
   do {                                             \
     hipError_t e__ = hipGetLastError();            \

@@ -25,7 +25,7 @@ namespace {
 
 constexpr int NO_PAGE = -1;
 constexpr int IA_HOST_ERROR = -2;
-constexpr int KIND_FULL = 0, KIND_WINDOW = 1;
+constexpr int KIND_FULL = 0, KIND_WINDOW = 1, KIND_CHUNK = 2;
 
 struct Pool {
   int num_pages = 0;
@@ -128,7 +128,7 @@ int ia_pool_is_used(void* h, int page) {
 }
 
 // ------------------------------------------------------------------------------------------- the cache
-// kinds[g]: 0 = all keys, 1 = a window of windows[g] keys.  Every group has num_pages pages of page_size.
+// kinds[g]: 0 = all keys, 1 = a window of windows[g] keys, 2 = chunks of windows[g] positions (a query sees its own chunk).  Every group has num_pages pages of page_size.
 void* ia_cache_create(int n_groups, const int* kinds, const int* windows, int page_size, int num_pages, int num_slots) {
   if (n_groups < 0 || page_size <= 0 || num_pages <= 0 || num_slots < 0) return nullptr;
   Cache* c = new Cache();
@@ -258,9 +258,12 @@ int ia_cache_commit(void* h, int64_t req, int64_t n_new) {
     Group& g = c->groups[gi];
     Table& t = g.tables[req];
     t.num_tokens += n_new;
-    if (g.kind == KIND_WINDOW && g.window > 0) {
-      // the next query stands at position num_tokens and sees keys >= num_tokens - window + 1
-      const int64_t first_needed = std::max<int64_t>(0, t.num_tokens - g.window + 1) / g.page_size;
+    if ((g.kind == KIND_WINDOW || g.kind == KIND_CHUNK) && g.window > 0) {
+      // the next query stands at position num_tokens and sees keys >= num_tokens - window + 1 (a window), or
+      // the keys of its own chunk of `window` positions, from floor(num_tokens / window) * window on (chunks)
+      const int64_t first_key = g.kind == KIND_WINDOW ? std::max<int64_t>(0, t.num_tokens - g.window + 1)
+                                                      : t.num_tokens / g.window * g.window;
+      const int64_t first_needed = first_key / g.page_size;
       const int stop = (int)std::min<int64_t>(first_needed, (int64_t)t.pages.size());
       while (t.first_live < stop) {
         const int p = t.pages[(size_t)t.first_live];

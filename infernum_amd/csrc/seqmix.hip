@@ -1,0 +1,451 @@
+// Kernels for mixers that carry a little state from token to token beside (or in place of) the paged cache:
+//
+//   ia_causal_conv         a short causal convolution over time on every channel, the last taps-1 inputs of every
+//                          request kept in its state slot (fp32), an optional bias on the input (a projection's),
+//                          an optional bias on the output and an optional silu
+//   ia_conv_state_update   the state of that convolution after a step
+//   ia_qk_prepare          query and key heads between projection and attention: an RMS norm per head (one weight
+//                          for all heads), rotation of neighbouring or half-split pairs with a factor on sine and
+//                          cosine, the keys to their pages, and as values either the value heads of the row or the
+//                          key heads as they came in
+//   ia_ssd_scan            the selective state-space recurrence  S <- a S + dt B x^T,  y = S^T C + D x  per head,
+//                          the state [N, P] of every request in its slot (fp32)
+//   ia_gated_group_norm    y * silu(z), then an RMS norm in equal parts of the row, times a weight
+//   ia_concat_cast         rows [cast(a) | b]: the operand of a product over two streams side by side
+//   ia_stream_add         the fp32 stream += a tensor or the partial sums of a split product
+//   ia_add_bias, ia_softcap
+//
+// Everything between the loads and the stores is fp32: sums of squares, angles, decays, step sizes, the state.
+// A row's result depends on its request's earlier tokens alone, in a fixed order of additions, so it is the same
+// bits however a prompt is cut into steps and whatever else is in the batch.
+#include "common.h"
+
+// ------------------------------------------------------------------------------------------ convolution
+// u [N, >= C] (stride u_stride), state [slots, taps-1, C] fp32: state[slot][j] is the input at position
+// ctx - (taps-1) + j of the request (zero before its start: a slot is cleared when it is taken).
+// y[t] = b_out + sum_j w[c, j] (u[t - (taps-1) + j] + b_in), j ascending.
+template <typename TU, typename TY>
+__global__ __launch_bounds__(256) void causal_conv_kernel(
+    const TU* __restrict__ u, int u_stride, const float* __restrict__ bias_in, const float* __restrict__ w,
+    const float* __restrict__ bias_out, int act, TY* __restrict__ y, int y_stride, const float* __restrict__ state,
+    long state_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_starts,
+    const int* __restrict__ state_slots, int N, int C, int taps) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (r >= N || c >= C) return;
+  const int s = token_seq[r];
+  const int i = r - seq_starts[s];
+  const float* st = state + (size_t)state_slots[s] * state_stride;
+  const float b_in = bias_in ? bias_in[c] : 0.f;
+  float acc = bias_out ? bias_out[c] : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int lag = taps - 1 - j;
+    float v;
+    if (i - lag >= 0)
+      v = to_float(u[(size_t)(r - lag) * u_stride + c]) + b_in;
+    else
+      v = st[(size_t)(i - lag + taps - 1) * C + c];
+    acc = __builtin_fmaf(w[(size_t)c * taps + j], v, acc);
+  }
+  if (act == 1) acc = acc / (1.f + expf(-acc));
+  y[(size_t)r * y_stride + c] = from_float<TY>(acc);
+}
+
+// After the step: state[slot][j] <- the input at position ctx + q - (taps-1) + j, from this step's rows or from the
+// old state (read in ascending j before the places are written: a thread owns its channel's taps-1 values).
+template <typename TU>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    const TU* __restrict__ u, int u_stride, const float* __restrict__ bias_in, float* __restrict__ state,
+    long state_stride, const int* __restrict__ seq_starts, const int* __restrict__ state_slots, int B, int C, int taps) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (s >= B || c >= C) return;
+  const int first = seq_starts[s], q = seq_starts[s + 1] - first;
+  float* st = state + (size_t)state_slots[s] * state_stride;
+  const float b_in = bias_in ? bias_in[c] : 0.f;
+  for (int j = 0; j < taps - 1; ++j) {
+    const int i = q - (taps - 1) + j;          // row of the request in this step, negative: before it
+    float v;
+    if (i >= 0)
+      v = to_float(u[(size_t)(first + i) * u_stride + c]) + b_in;
+    else
+      v = st[(size_t)(j + q) * C + c];
+    st[(size_t)j * C + c] = v;
+  }
+}
+
+extern "C" int ia_causal_conv(const void* u, int u_code, int u_stride, const float* bias_in, const float* w,
+                              const float* bias_out, int act, void* y, int y_code, int y_stride, const float* state,
+                              long state_stride, const int* token_seq, const int* seq_starts, const int* state_slots, int N, int C,
+                              int taps, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!u || !w || !y || !state || !token_seq || !seq_starts || !state_slots || C <= 0 || taps < 1 || u_stride < C ||
+      y_stride < C || N < 0 || N > 65535 || state_stride < (long)(taps - 1) * C || (act != 0 && act != 1))
+    return IA_ERR_BAD_ARG;
+  const dim3 grid((unsigned)((C + 255) / 256), (unsigned)N);
+#define IA_CONV(TU, TY)                                                                                          \
+  causal_conv_kernel<TU, TY><<<grid, 256, 0, stream>>>((const TU*)u, u_stride, bias_in, w, bias_out, act, (TY*)y, \
+                                                       y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps)
+  if (u_code == IA_F32 && y_code == IA_F32) IA_CONV(float, float);
+  else if (u_code == IA_BF16 && y_code == IA_BF16) IA_CONV(bf16_t, bf16_t);
+  else if (u_code == IA_F32 && y_code == IA_BF16) IA_CONV(float, bf16_t);
+  else if (u_code == IA_BF16 && y_code == IA_F32) IA_CONV(bf16_t, float);
+  else return IA_ERR_BAD_ARG;
+#undef IA_CONV
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+extern "C" int ia_conv_state_update(const void* u, int u_code, int u_stride, const float* bias_in, float* state,
+                                    long state_stride, const int* seq_starts, const int* state_slots, int B, int C, int taps,
+                                    hipStream_t stream) {
+  if (B == 0 || taps <= 1) return IA_OK;
+  if (!u || !state || !seq_starts || !state_slots || C <= 0 || u_stride < C || B < 0 || B > 65535 ||
+      state_stride < (long)(taps - 1) * C)
+    return IA_ERR_BAD_ARG;
+  const dim3 grid((unsigned)((C + 255) / 256), (unsigned)B);
+  if (u_code == IA_F32)
+    conv_state_update_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, u_stride, bias_in, state, state_stride,
+                                                             seq_starts, state_slots, B, C, taps);
+  else if (u_code == IA_BF16)
+    conv_state_update_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, u_stride, bias_in, state, state_stride,
+                                                              seq_starts, state_slots, B, C, taps);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ------------------------------------------------------------------------------------------ queries and keys
+// One wave per (token, head).  Rows of x: nh query heads, nkv key heads, and nkv value heads when the values are
+// not the keys.  pairing 0: value i with value i + rot/2; 1: value 2i with value 2i+1.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_prepare_kernel(
+    const T* __restrict__ x, int x_stride, T* __restrict__ q_out, int q_stride, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float eps, const int* __restrict__ positions, const int* __restrict__ slots,
+    const void* __restrict__ freq, int freq_f64, int rot, int pairing, float magnitude, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int N, int nh, int nkv, int d, int page_size, int num_pages, int values_are_keys) {
+  const int lane = threadIdx.x & 63;
+  const int heads = nh + nkv;
+  const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= (long)N * heads) return;
+  const int t = (int)(item / heads), hd = (int)(item % heads);
+  const bool is_key = hd >= nh;
+  if (is_key && !k_pages) return;
+  const T* src = x + (size_t)t * x_stride + (size_t)hd * d;
+  const float* wn = is_key ? k_norm : q_norm;
+  // the norm: sum of squares over the head, lanes strided, joined across the wave in a fixed order
+  float ss = 0.f;
+  for (int i = lane; i < d; i += 64) {
+    const float v = to_float(src[i]);
+    ss = __builtin_fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = wn ? 1.0f / sqrtf(ss / (float)d + eps) : 1.0f;
+  const int pos = positions[t];
+  T* dst;
+  if (is_key) {
+    const int slot = slots[t];
+    const int page = slot / page_size, off = slot - page * page_size;
+    if (page < 0 || page >= num_pages) return;
+    const int g = hd - nh;
+    dst = k_pages + (((size_t)page * nkv + g) * page_size + off) * d;
+    // the values: the value head of the row, or the key head as it came in; transposed within the page
+    const T* vsrc = values_are_keys ? src : x + (size_t)t * x_stride + (size_t)(heads + g) * d;
+    T* vdst = v_pages + ((size_t)page * nkv + g) * (size_t)d * page_size + off;
+    for (int i = lane; i < d; i += 64) vdst[(size_t)i * page_size] = vsrc[i];
+  } else {
+    dst = q_out + (size_t)t * q_stride + (size_t)hd * d;
+  }
+  const int half = rot >> 1;
+  // rotated pairs first, then the values that pass
+  for (int p = lane; p < half; p += 64) {
+    const int ia = pairing ? 2 * p : p, ib = pairing ? 2 * p + 1 : p + half;
+    float a = to_float(src[ia]) * inv, b = to_float(src[ib]) * inv;
+    if (wn) { a *= wn[ia]; b *= wn[ib]; }
+    float sn, cs, lo, hi;
+    rope_sincos(pos, freq, freq_f64, p, sn, cs);
+    sn *= magnitude;
+    cs *= magnitude;
+    rope_pair(a, b, cs, sn, lo, hi);
+    dst[ia] = from_float<T>(lo);
+    dst[ib] = from_float<T>(hi);
+  }
+  for (int i = rot + lane; i < d; i += 64) {
+    float a = to_float(src[i]) * inv;
+    if (wn) a *= wn[i];
+    dst[i] = from_float<T>(a);
+  }
+}
+
+extern "C" int ia_qk_prepare(const void* x, int code, int x_stride, void* q_out, int q_stride, const float* q_norm,
+                             const float* k_norm, float eps, const int* positions, const int* slots, const void* freq,
+                             int freq_f64, int rot, int pairing, float magnitude, void* k_pages, void* v_pages, int N,
+                             int nh, int nkv, int d, int page_size, int num_pages, int values_are_keys,
+                             hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  const int write = k_pages != nullptr;
+  if (!x || !q_out || !positions || N < 0 || nh <= 0 || nkv < 0 || d <= 0 || rot < 0 || rot > d || (rot & 1) ||
+      (rot > 0 && !freq) || (write && (!v_pages || !slots || page_size <= 0 || num_pages <= 0)) ||
+      x_stride < (nh + (write ? (values_are_keys ? nkv : 2 * nkv) : 0)) * d || q_stride < nh * d ||
+      (q_norm == nullptr) != (k_norm == nullptr))
+    return IA_ERR_BAD_ARG;
+  // the rotation reads its pair from the source and writes both places: in place only where source and
+  // destination are the same element for element (q_out == x with equal strides), which this launch allows
+  const long items = (long)N * (nh + nkv);
+  const unsigned grid = (unsigned)((items + 3) / 4);
+  if (code == IA_F32)
+    qk_prepare_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (float*)q_out, q_stride, q_norm, k_norm,
+                                                      eps, positions, slots, freq, freq_f64, rot, pairing, magnitude,
+                                                      (float*)k_pages, (float*)v_pages, N, nh, nkv, d, page_size,
+                                                      num_pages, values_are_keys);
+  else if (code == IA_BF16)
+    qk_prepare_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_stride, (bf16_t*)q_out, q_stride, q_norm,
+                                                       k_norm, eps, positions, slots, freq, freq_f64, rot, pairing,
+                                                       magnitude, (bf16_t*)k_pages, (bf16_t*)v_pages, N, nh, nkv, d,
+                                                       page_size, num_pages, values_are_keys);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ------------------------------------------------------------------------------------------ the recurrence
+// One workgroup per (request, head).  Thread (part, p) keeps the state values S[n][p] for n = part, part + parts,
+// ... in registers over the request's tokens of this step; per token the parts' shares of y[p] = sum_n S[n][p] C[n]
+// meet in LDS and are added in the order of the parts.  xbc rows: [x: nh P | B: G N | C: G N] after their
+// convolution; dt rows: nh raw step sizes.  y [T, nh P] fp32.
+template <typename T, int KMAX>
+__global__ __launch_bounds__(256) void ssd_scan_kernel(
+    const T* __restrict__ xbc, int xbc_stride, const T* __restrict__ dt_raw, int dt_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ skip,
+    float* __restrict__ state, long state_stride, float* __restrict__ y, const int* __restrict__ seq_starts,
+    const int* __restrict__ state_slots, int nh, int P, int Ns, int G, int parts) {
+  extern __shared__ float lds[];
+  float* bc = lds;                       // [2][2 Ns]: B and C of a token, two tokens in turn
+  float* ysum = lds + 4 * Ns;            // [parts][P]
+  const int s = blockIdx.y, hd = blockIdx.x;
+  const int first = seq_starts[s], q = seq_starts[s + 1] - first;
+  const int g = hd / (nh / G);
+  const int tid = threadIdx.x;
+  const int p = tid % P, part = tid / P;
+  const bool live = part < parts;
+  float* S = state + (size_t)state_slots[s] * state_stride + (size_t)hd * Ns * P;
+  float reg[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int n = part + k * parts;
+    reg[k] = (live && n < Ns) ? S[(size_t)n * P + p] : 0.f;
+  }
+  const float A = -expf(a_log[hd]);
+  const float bias = dt_bias[hd], D = skip[hd];
+  const size_t b_col = (size_t)nh * P + (size_t)g * Ns, c_col = (size_t)nh * P + (size_t)G * Ns + (size_t)g * Ns;
+  for (int i = 0; i < q; ++i) {
+    const size_t row = (size_t)(first + i);
+    float* cur = bc + (i & 1) * 2 * Ns;
+    for (int n = tid; n < 2 * Ns; n += blockDim.x)
+      cur[n] = to_float(xbc[row * xbc_stride + (n < Ns ? b_col + n : c_col + (n - Ns))]);
+    const float z = to_float(dt_raw[row * dt_stride + hd]) + bias;
+    const float dt = z > 20.f ? z : log1pf(expf(z));
+    const float decay = expf(A * dt);
+    const float xv = live ? to_float(xbc[row * xbc_stride + (size_t)hd * P + p]) : 0.f;
+    const float dx = dt * xv;
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int n = part + k * parts;
+      if (n < Ns) {
+        reg[k] = __builtin_fmaf(decay, reg[k], dx * cur[n]);
+        acc = __builtin_fmaf(reg[k], cur[Ns + n], acc);
+      }
+    }
+    if (live) ysum[part * P + p] = acc;
+    __syncthreads();
+    if (part == 0) {
+      float t = ysum[p];
+      for (int k = 1; k < parts; ++k) t += ysum[k * P + p];
+      y[row * ((size_t)nh * P) + (size_t)hd * P + p] = __builtin_fmaf(D, xv, t);
+    }
+    // the next token's B and C go to the other half of bc; ysum is read before the next token's barrier pair ends
+  }
+  if (live) {
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int n = part + k * parts;
+      if (n < Ns) S[(size_t)n * P + p] = reg[k];
+    }
+  }
+}
+
+extern "C" int ia_ssd_scan(const void* xbc, int code, int xbc_stride, const void* dt_raw, int dt_stride,
+                           const float* dt_bias, const float* a_log, const float* skip, float* state, long state_stride,
+                           float* y, const int* seq_starts, const int* state_slots, int B, int nh, int P, int Ns, int G,
+                           hipStream_t stream) {
+  if (B == 0) return IA_OK;
+  if (!xbc || !dt_raw || !dt_bias || !a_log || !skip || !state || !y || !seq_starts || !state_slots || B < 0 ||
+      B > 65535 || nh <= 0 || P <= 0 || P > 256 || Ns <= 0 || G <= 0 || nh % G || xbc_stride < nh * P + 2 * G * Ns ||
+      dt_stride < nh || state_stride < (long)nh * Ns * P)
+    return IA_ERR_BAD_ARG;
+  int parts = 256 / P;
+  if (parts > Ns) parts = Ns;
+  const int per = (Ns + parts - 1) / parts;
+  if (per > 128) return IA_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)nh, (unsigned)B);
+  const size_t lds = sizeof(float) * (4 * (size_t)Ns + (size_t)parts * P);
+  if (lds > 64 * 1024) return IA_ERR_UNSUPPORTED;
+#define IA_SCAN(T, KM)                                                                                            \
+  ssd_scan_kernel<T, KM><<<grid, 256, lds, stream>>>((const T*)xbc, xbc_stride, (const T*)dt_raw, dt_stride, dt_bias, \
+                                                     a_log, skip, state, state_stride, y, seq_starts, state_slots, nh, P, Ns, G,  \
+                                                     parts)
+#define IA_SCAN_K(T)                       \
+  do {                                     \
+    if (per <= 8) IA_SCAN(T, 8);           \
+    else if (per <= 16) IA_SCAN(T, 16);    \
+    else if (per <= 32) IA_SCAN(T, 32);    \
+    else if (per <= 64) IA_SCAN(T, 64);    \
+    else IA_SCAN(T, 128);                  \
+  } while (0)
+  if (code == IA_F32) IA_SCAN_K(float);
+  else if (code == IA_BF16) IA_SCAN_K(bf16_t);
+  else return IA_ERR_BAD_ARG;
+#undef IA_SCAN_K
+#undef IA_SCAN
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ------------------------------------------------------------------------------------------ gate and norm
+// One workgroup per (row, part): out = unit_rms(y * silu(z)) * w over the part's `size` values.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z,
+                                                               int z_stride, const float* __restrict__ w,
+                                                               T* __restrict__ out, int inner, int size, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.y, part = blockIdx.x;
+  const size_t base = (size_t)part * size;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < size; i += 256) {
+    const float g = to_float(z[(size_t)r * z_stride + base + i]);
+    const float v = y[(size_t)r * inner + base + i] * (g / (1.f + expf(-g)));
+    ss = __builtin_fmaf(v, v, ss);
+  }
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+  for (int i = threadIdx.x; i < size; i += 256) {
+    const float g = to_float(z[(size_t)r * z_stride + base + i]);
+    const float v = y[(size_t)r * inner + base + i] * (g / (1.f + expf(-g)));
+    out[(size_t)r * inner + base + i] = from_float<T>(v * inv * w[base + i]);
+  }
+}
+
+extern "C" int ia_gated_group_norm(const float* y, const void* z, int code, int z_stride, const float* w, void* out,
+                                   int N, int inner, int groups, float eps, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!y || !z || !w || !out || N < 0 || N > 65535 || inner <= 0 || groups <= 0 || inner % groups || z_stride < inner)
+    return IA_ERR_BAD_ARG;
+  const dim3 grid((unsigned)groups, (unsigned)N);
+  if (code == IA_F32)
+    gated_group_norm_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)z, z_stride, w, (float*)out, inner,
+                                                            inner / groups, eps);
+  else if (code == IA_BF16)
+    gated_group_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>(y, (const bf16_t*)z, z_stride, w, (bf16_t*)out, inner,
+                                                             inner / groups, eps);
+  else
+    return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// ------------------------------------------------------------------------------------------ small row kernels
+// out [N, 2 W] = [cast(a [N, W] fp32) | b [N, W]]
+template <typename T>
+__global__ __launch_bounds__(256) void concat_cast_kernel(const float* __restrict__ a, const T* __restrict__ b,
+                                                          T* __restrict__ out, size_t n, int W) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const size_t r = i / W, c = i - r * W;
+    out[r * 2 * W + c] = from_float<T>(a[i]);
+    out[r * 2 * W + W + c] = b[i];
+  }
+}
+
+extern "C" int ia_concat_cast(const float* a, const void* b, void* out, int code, int N, int W, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!a || !b || !out || N < 0 || W <= 0) return IA_ERR_BAD_ARG;
+  const size_t n = (size_t)N * W;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (code == IA_F32) concat_cast_kernel<float><<<grid, 256, 0, stream>>>(a, (const float*)b, (float*)out, n, W);
+  else if (code == IA_BF16) concat_cast_kernel<bf16_t><<<grid, 256, 0, stream>>>(a, (const bf16_t*)b, (bf16_t*)out, n, W);
+  else return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// h [N, H] fp32 += delta, a tensor [N, H] or a stack of partial sums [splits, N, H], added in the order of their index
+template <typename T>
+__global__ __launch_bounds__(256) void stream_add_kernel(float* __restrict__ h, const T* __restrict__ delta, int splits,
+                                                         size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) h[i] += load_split_sum(delta + i, splits, n);
+}
+
+extern "C" int ia_stream_add(float* h, const void* delta, int code, int splits, int N, int H, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!h || !delta || N < 0 || H <= 0 || splits < 1) return IA_ERR_BAD_ARG;
+  const size_t n = (size_t)N * H;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (code == IA_F32) stream_add_kernel<float><<<grid, 256, 0, stream>>>(h, (const float*)delta, splits, n);
+  else if (code == IA_BF16) stream_add_kernel<bf16_t><<<grid, 256, 0, stream>>>(h, (const bf16_t*)delta, splits, n);
+  else return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// y [N, C] += bias (fp32 vector), rounded once
+template <typename T>
+__global__ __launch_bounds__(256) void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, size_t n, int C) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    y[i] = from_float<T>(to_float(y[i]) + bias[i % C]);
+}
+
+extern "C" int ia_add_bias(void* y, int code, const float* bias, int N, int C, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!y || !bias || N < 0 || C <= 0) return IA_ERR_BAD_ARG;
+  const size_t n = (size_t)N * C;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (code == IA_F32) add_bias_kernel<float><<<grid, 256, 0, stream>>>((float*)y, bias, n, C);
+  else if (code == IA_BF16) add_bias_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)y, bias, n, C);
+  else return IA_ERR_BAD_ARG;
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+// x <- cap * tanh(x / cap), fp32 in place
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  const float inv = 1.0f / cap;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) x[i] = cap * tanhf(x[i] * inv);
+}
+
+extern "C" int ia_softcap(float* x, int rows, int cols, float cap, hipStream_t stream) {
+  if (rows == 0) return IA_OK;
+  if (!x || rows < 0 || cols <= 0 || !(cap > 0.f)) return IA_ERR_BAD_ARG;
+  const size_t n = (size_t)rows * cols;
+  const unsigned grid = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  softcap_kernel<<<grid, 256, 0, stream>>>(x, n, cap);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
+#include "op_call.h"
+IA_OP(ia_causal_conv)
+IA_OP(ia_conv_state_update)
+IA_OP(ia_qk_prepare)
+IA_OP(ia_ssd_scan)
+IA_OP(ia_gated_group_norm)
+IA_OP(ia_concat_cast)
+IA_OP(ia_stream_add)
+IA_OP(ia_add_bias)
+IA_OP(ia_softcap)

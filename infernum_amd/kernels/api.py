@@ -911,8 +911,8 @@ def prefill_launch_shape(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_l
     for q, c in zip(q_lens, ctx_lens):
         for first in range(0, q, 64):           # a block of 64 rows sees the keys up to its last row, or a window's worth
             keys = c + min(q, first + 64)
-            if window > 0:
-                keys = min(keys, window + 64)
+            if window:                          # a sliding window, or (negative) chunks of that many positions
+                keys = min(keys, abs(window) + 64)
             tiles += 1
             total += keys
             longest = max(longest, keys)
@@ -929,6 +929,176 @@ def prefill_launch_shape(nh: int, nkv: int, d: int, q_lens: Sequence[int], ctx_l
     if hpw == 4 and workgroups <= cus and longest * tiles >= 1.5 * total:
         hpw = 2
     return hpw
+
+
+# ------------------------------------------------------------- mixers with a little state from token to token
+CONV_ACTIVATIONS = {None: 0, "silu": 1}
+PAIRINGS = {"half": 0, "neighbours": 1}
+
+
+def _f32(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is not None:
+        _need(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n, f"{what}: {n} fp32 values")
+
+
+def _rows(t: torch.Tensor, cols: int, what: str) -> None:
+    _need(t.is_cuda and t.dim() == 2 and t.stride(1) == 1 and t.shape[1] >= cols and t.dtype in DTYPE_CODE,
+          f"{what}: rows of at least {cols} values, fp32 or bf16")
+
+
+def _state_rows(state: torch.Tensor, need: int, what: str) -> int:
+    """``state`` [slots, per slot] fp32, a slot's values consecutive: the slot's stride in floats."""
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state.shape[1] >= need, f"{what}: state [slots, >= {need}] fp32")
+    return int(state.stride(0))
+
+
+def causal_conv(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, ctx_token_seq: torch.Tensor,
+                seq_starts: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                bias_in: Optional[torch.Tensor] = None, bias_out: Optional[torch.Tensor] = None,
+                activation: Optional[str] = None) -> torch.Tensor:
+    """out[t, c] = act(bias_out[c] + sum_j w[c, j] (u[t - (taps-1) + j, c] + bias_in[c])) over each request's own
+    tokens; the inputs before this step's rows come from ``state`` [slots, >= (taps-1) C] fp32 (the request's last
+    taps-1 inputs, zero before its start).  ``u`` and ``out`` may be column ranges of wider rows.  The state is
+    left as it was: :func:`conv_state_update` moves it on."""
+    N, (C, taps) = u.shape[0], w.shape
+    _rows(u, C, "causal_conv input")
+    _rows(out, C, "causal_conv output")
+    _need(out.shape[0] == N and u.shape[1] == C and out.shape[1] == C, "causal_conv: u and out are [N, C]")
+    _f32(w, C * taps, "causal_conv weight")
+    _f32(bias_in, C, "causal_conv input bias")
+    _f32(bias_out, C, "causal_conv output bias")
+    stride = _state_rows(state, (taps - 1) * C, "causal_conv")
+    _i32(ctx_token_seq, N, "causal_conv token_seq")
+    _ok(_core().ia_causal_conv(_p(u), DTYPE_CODE[u.dtype], u.stride(0), _p(bias_in), _p(w), _p(bias_out),
+                               CONV_ACTIVATIONS[activation], _p(out), DTYPE_CODE[out.dtype], out.stride(0), _p(state),
+                               ctypes.c_long(stride), _p(ctx_token_seq), _p(seq_starts), _p(state_slots), N, C, taps,
+                               _stream()), "causal_conv")
+    return out
+
+
+def conv_state_update(u: torch.Tensor, taps: int, state: torch.Tensor, seq_starts: torch.Tensor,
+                      state_slots: torch.Tensor, bias_in: Optional[torch.Tensor] = None) -> None:
+    """After :func:`causal_conv`: every request's state becomes its last taps-1 inputs, this step's included."""
+    C, B = u.shape[1], state_slots.numel()
+    _rows(u, C, "conv_state_update input")
+    _f32(bias_in, C, "conv_state_update input bias")
+    stride = _state_rows(state, (taps - 1) * C, "conv_state_update")
+    _need(seq_starts.numel() >= B + 1, "conv_state_update: seq_starts holds B + 1 rows")
+    _ok(_core().ia_conv_state_update(_p(u), DTYPE_CODE[u.dtype], u.stride(0), _p(bias_in), _p(state),
+                                     ctypes.c_long(stride), _p(seq_starts), _p(state_slots), B, C, int(taps), _stream()),
+        "conv_state_update")
+
+
+def qk_prepare(x: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, d: int, positions: torch.Tensor,
+               q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, eps: float = 0.0,
+               freq: Optional[torch.Tensor] = None, rot: int = 0, pairing: str = "half", magnitude: float = 1.0,
+               slots: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
+               v_pages: Optional[torch.Tensor] = None, values_are_keys: bool = False) -> torch.Tensor:
+    """Query and key heads between projection and attention.  ``x`` [N, (nh + nkv (+ nkv)) d]: nh query heads,
+    nkv key heads, and nkv value heads unless ``values_are_keys`` (then a key head as it comes in is its value).
+    Per head: RMS norm over d with one weight for all heads (when given), rotation of the first ``rot`` values
+    (``pairing`` "half": value i with i + rot/2; "neighbours": 2i with 2i+1) with sine and cosine times
+    ``magnitude``.  Queries go to ``q_out`` [N, nh d], keys and values to their pages at ``slots``."""
+    N = x.shape[0]
+    write = k_pages is not None
+    _rows(x, (nh + (nkv if values_are_keys else 2 * nkv) * int(write)) * d, "qk_prepare input")
+    _rows(q_out, nh * d, "qk_prepare q_out")
+    _need(q_out.dtype == x.dtype and q_out.shape[0] == N, "qk_prepare: q_out [N, nh d] of the input's dtype")
+    _f32(q_norm, d, "qk_prepare q_norm")
+    _f32(k_norm, d, "qk_prepare k_norm")
+    _i32(positions, N, "qk_prepare positions")
+    if rot:
+        _need(freq is not None and freq.is_cuda and freq.dtype in (torch.float32, torch.float64)
+              and freq.numel() == rot // 2 and rot % 2 == 0 and rot <= d, "qk_prepare: rot/2 frequencies, rot even, <= d")
+    ps = num_pages = 0
+    if write:
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        _need(slots is not None and v_pages is not None and k_pages.dtype == x.dtype and v_pages.dtype == x.dtype
+              and tuple(k_pages.shape) == (num_pages, nkv, ps, d) and tuple(v_pages.shape) == (num_pages, nkv, d, ps)
+              and k_pages.is_contiguous() and v_pages.is_contiguous(),
+              "qk_prepare: key pages [num_pages, nkv, page_size, d], value pages [num_pages, nkv, d, page_size]")
+        _i32(slots, N, "qk_prepare slots")
+    _ok(_core().ia_qk_prepare(_p(x), DTYPE_CODE[x.dtype], x.stride(0), _p(q_out), q_out.stride(0), _p(q_norm), _p(k_norm),
+                              ctypes.c_float(eps), _p(positions), _p(slots), _p(freq if rot else None),
+                              1 if (rot and freq.dtype == torch.float64) else 0, int(rot), PAIRINGS[pairing],
+                              ctypes.c_float(magnitude), _p(k_pages), _p(v_pages), N, nh, nkv if write else 0, d, ps,
+                              num_pages, int(bool(values_are_keys)), _stream()), "qk_prepare")
+    return q_out
+
+
+def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, skip: torch.Tensor,
+             state: torch.Tensor, y: torch.Tensor, seq_starts: torch.Tensor, state_slots: torch.Tensor, nh: int, P: int,
+             Ns: int, G: int) -> torch.Tensor:
+    """Per request and head, over the request's rows in order:  dt = softplus(dt_raw + dt_bias),
+    S <- exp(-exp(a_log) dt) S + dt B x^T,  y = S^T C + skip x.  ``xbc`` rows [x: nh P | B: G Ns | C: G Ns];
+    ``state`` [slots, >= nh Ns P] fp32 is read and left moved on; ``y`` [N, nh P] fp32."""
+    N, B = xbc.shape[0], state_slots.numel()
+    _rows(xbc, nh * P + 2 * G * Ns, "ssd_scan xbc")
+    _rows(dt_raw, nh, "ssd_scan dt")
+    _need(dt_raw.dtype == xbc.dtype and dt_raw.shape[0] == N, "ssd_scan: dt rows of xbc's dtype")
+    for t, what in ((dt_bias, "dt_bias"), (a_log, "a_log"), (skip, "skip")):
+        _f32(t, nh, "ssd_scan " + what)
+    _need(y.is_cuda and y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (N, nh * P),
+          "ssd_scan: y [N, nh P] fp32")
+    stride = _state_rows(state, nh * Ns * P, "ssd_scan")
+    _ok(_core().ia_ssd_scan(_p(xbc), DTYPE_CODE[xbc.dtype], xbc.stride(0), _p(dt_raw), dt_raw.stride(0), _p(dt_bias),
+                            _p(a_log), _p(skip), _p(state), ctypes.c_long(stride), _p(y), _p(seq_starts), _p(state_slots),
+                            B, nh, P, Ns, G, _stream()), "ssd_scan")
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                     out: torch.Tensor) -> torch.Tensor:
+    """out = unit_rms(y * silu(z)) * w, the root mean square taken over each of ``groups`` equal parts of a row."""
+    N, inner = y.shape
+    _need(y.is_cuda and y.dtype == torch.float32 and y.is_contiguous(), "gated_group_norm: y [N, inner] fp32")
+    _rows(z, inner, "gated_group_norm gate")
+    _f32(w, inner, "gated_group_norm weight")
+    _need(out.is_cuda and out.is_contiguous() and tuple(out.shape) == (N, inner) and out.dtype == z.dtype
+          and inner % groups == 0, "gated_group_norm: out [N, inner] of the gate's dtype, inner a multiple of groups")
+    _ok(_core().ia_gated_group_norm(_p(y), _p(z), DTYPE_CODE[z.dtype], z.stride(0), _p(w), _p(out), N, inner, int(groups),
+                                    ctypes.c_float(eps), _stream()), "gated_group_norm")
+    return out
+
+
+def concat_cast(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[N, 2 W] rows [cast(a) | b]: a fp32 [N, W], b [N, W] in the result's dtype."""
+    N, W = a.shape
+    _need(a.is_cuda and a.dtype == torch.float32 and a.is_contiguous() and b.is_cuda and b.is_contiguous()
+          and tuple(b.shape) == (N, W) and b.dtype in DTYPE_CODE, "concat_cast: a fp32 [N, W], b [N, W]")
+    if out is None:
+        out = torch.empty((N, 2 * W), dtype=b.dtype, device=b.device)
+    _need(out.is_contiguous() and tuple(out.shape) == (N, 2 * W) and out.dtype == b.dtype, "concat_cast: out [N, 2 W]")
+    _ok(_core().ia_concat_cast(_p(a), _p(b), _p(out), DTYPE_CODE[b.dtype], N, W, _stream()), "concat_cast")
+    return out
+
+
+def stream_add(h: torch.Tensor, delta) -> torch.Tensor:
+    """h [N, H] fp32 += delta: a tensor [N, H], or a :class:`SplitSum` whose parts are added in the order of their index."""
+    parts = delta.parts if isinstance(delta, SplitSum) else delta
+    splits = parts.shape[0] if isinstance(delta, SplitSum) else 1
+    _need(h.is_cuda and h.dtype == torch.float32 and h.is_contiguous() and parts.is_cuda and parts.is_contiguous()
+          and parts.dtype in DTYPE_CODE and parts.numel() == splits * h.numel(), "stream_add: h fp32 [N, H], delta of its shape")
+    _ok(_core().ia_stream_add(_p(h), _p(parts), DTYPE_CODE[parts.dtype], splits, h.shape[0], h.shape[1], _stream()),
+        "stream_add")
+    return h
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y [N, C] += bias [C] (fp32), in place."""
+    _need(y.is_cuda and y.is_contiguous() and y.dim() == 2 and y.dtype in DTYPE_CODE, "add_bias: y [N, C]")
+    _f32(bias, y.shape[1], "add_bias bias")
+    _ok(_core().ia_add_bias(_p(y), DTYPE_CODE[y.dtype], _p(bias), y.shape[0], y.shape[1], _stream()), "add_bias")
+    return y
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap tanh(logits / cap), fp32 in place."""
+    _need(logits.is_cuda and logits.dtype == torch.float32 and logits.is_contiguous() and logits.dim() == 2 and cap > 0,
+          "softcap: logits fp32 [R, V], cap positive")
+    _ok(_core().ia_softcap(_p(logits), logits.shape[0], logits.shape[1], ctypes.c_float(cap), _stream()), "softcap")
+    return logits
 
 
 # ------------------------------------------------------------------------- sampling

@@ -50,7 +50,7 @@ class Attention(Mixer):
     def __init__(self, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[Mapping[str, Any]] = None, window: Optional[int] = None,
                  scale: Optional[float] = None, kernels: str = "auto", init_std: float = 0.02,
-                 qk_transform: Optional[Mapping[str, Any]] = None):
+                 qk_transform: Optional[Mapping[str, Any]] = None, chunk: Optional[int] = None):
         super().__init__(rt)
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
@@ -58,6 +58,12 @@ class Attention(Mixer):
             raise ValueError(f"head size {head_dim} is above {K.GENERIC_MAX_HEAD_DIM}, the largest the attention kernels take")
         self.hidden_size, self.nh, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
         self.window = int(window) if window else 0
+        # chunks of so many positions, counted from the request's start: a query sees the keys of its own chunk
+        self.chunk = int(chunk) if chunk else 0
+        if self.window < 0 or self.chunk < 0 or (self.window and self.chunk):
+            raise ValueError("attention takes a window or chunks, each positive, not both")
+        # what the kernels are told: 0 all keys, w > 0 a window of w keys, -c chunks of c positions
+        self.mask = self.window if self.window else -self.chunk
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         if kernels not in ("auto", "generic"):
             raise ValueError("kernels must be 'auto' or 'generic'")
@@ -82,6 +88,8 @@ class Attention(Mixer):
 
     # ---- what it needs ---------------------------------------------------
     def cache_spec(self) -> CacheSpec:
+        if self.chunk:                  # pages of chunks that every later query has left go back to the pool
+            return CacheSpec("chunk", self.nkv, self.d, self.chunk)
         return CacheSpec("window" if self.window else "full", self.nkv, self.d, self.window)
 
     def step_needs(self) -> Dict[str, Any]:
@@ -105,6 +113,8 @@ class Attention(Mixer):
         return own
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        if getattr(self.position, "magnitude", 1.0) != 1.0:
+            raise ValueError("this mixer's rotation has no factor on sine and cosine; 'conv_attention' has")
         wq, wk = tensors["q_proj.weight"], tensors["k_proj.weight"]
         perm = self.position.head_permutation()
         if perm is not None:
@@ -151,7 +161,7 @@ class Attention(Mixer):
             out = torch.empty((n, nh * d), dtype=dtype, device=cache.k_pages.device)
             K.attention_decode_rotating(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                                         ctx.slots[g] if cache.writable else None, cache.k_pages, cache.v_pages, out,
-                                        ctx.block_tables[g], nh, nkv, d, self.scale, self.window, ctx.max_total_len)
+                                        ctx.block_tables[g], nh, nkv, d, self.scale, self.mask, self._span(ctx.max_total_len))
             return out
         q_out = None
         if isinstance(qkv, K.SplitSum):
@@ -198,7 +208,7 @@ class Attention(Mixer):
         single tokens on the first rows and the one for portions of prompts on the rest (or the plain kernel on all
         rows).  Returns the buffer [N, nh d] of the attended rows."""
         from ..engine.program import NEVER, STREAM, Guard
-        nh, nkv, d, window, rt = self.nh, self.nkv, self.d, self.window, self.rt
+        nh, nkv, d, window, rt = self.nh, self.nkv, self.d, self.mask, self.rt
         k, v, g, writable = view.k_pages, view.v_pages, view.group, view.writable
         ps, num_pages = int(k.shape[2]), int(k.shape[0])
         inv_freq = self.position.inv_freq
@@ -220,26 +230,7 @@ class Attention(Mixer):
             records = T + 1024      # requests x parts of their keys: what fills the GPU, or the requests themselves
             part_o = program.buffer("attention.part_o", records * nh * d * 4)
             part_ml = program.buffer("attention.part_ml", records * nh * 2 * 4)
-            dev = rt.device
-
-            def parts_of_the_keys(ctx: StepContext) -> int:
-                nd = ctx.num_decode
-                if nd == 0:
-                    return 1
-                if ctx.block_tables[g].shape[1] * ps < ctx.max_total_len:
-                    raise K.KernelError("attention: the block tables are narrower than the longest request")
-                n = K.decode_splits(nd, nh, nkv, ctx.max_total_len, dev, d)
-                if nd * n > records:
-                    raise K.KernelError("attention: the parts of the keys do not fit the program's arena")
-                return n
-
-            def launch_shape(ctx: StepContext) -> int:
-                nd = ctx.num_decode
-                if ctx.num_seqs == nd:
-                    return 0
-                return K.prefill_launch_shape(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:], window, dev)
-            splits = program.scalar(("attention: parts of the keys", nh, nkv, g, ps), parts_of_the_keys)
-            shape = program.scalar(("attention: launch shape", nh, nkv, d, window), launch_shape)
+            splits, shape = self._attend_scalars(program, g, ps, records)
             tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
         for alt in qkv.alts:
             src, code, parts = alt.where, (K.DTYPE_CODE[torch.float32] if alt.splits else act), (alt.splits or 1)
@@ -255,41 +246,91 @@ class Attention(Mixer):
                        [src, code, parts, N, q, q_stride, act, program.positions, slots, inv_freq, f64,
                         k if writable else None, v if writable else None, N, row, nh, nkv, d, rot,
                         ps if writable else 0, num_pages if writable else 0, int(writable), STREAM], alt.when & separate)
-            if not mfma:
-                program.op("core", "ia_attention_generic",
-                           [q, q_stride, k, v, out, nh * d, act, program.token_seq, program.positions, bt, bt_cols, N, nh,
-                            nkv, d, ps, num_pages, scale, window, STREAM], alt.when & separate)
-                continue
-            program.op(lib, "ia_attn_decode",
-                       [q, q_stride, k, v, out, nh * d, part_o, part_ml, program.positions, bt, bt_cols, program.ND, nh,
-                        nkv, ps, num_pages, scale, window, splits, STREAM],
-                       alt.when & separate & Guard.between(program.ND, 1))
-            program.op(lib, "ia_attn_prefill",
-                       [q, q_stride, k, v, out, nh * d, program.seq_starts, program.seq_ctx, bt, bt_cols, tiles, num_tiles,
-                        nh, nkv, ps, num_pages, scale, window, shape, STREAM],
-                       alt.when & separate & Guard.between(program.NP, 1))
+            self.emit_attend(program, view, q, q_stride, alt.when & separate, out)
         return out
+
+    def _attend_scalars(self, program, g: int, ps: int, records: int):
+        """The two numbers that the host works out for the attention kernels once a step: into how many parts the
+        keys of single tokens are cut, and the launch shape of the kernel for portions of prompts."""
+        nh, nkv, d, window, dev = self.nh, self.nkv, self.d, self.mask, self.rt.device
+
+        def parts_of_the_keys(ctx: StepContext) -> int:
+            nd = ctx.num_decode
+            if nd == 0:
+                return 1
+            if ctx.block_tables[g].shape[1] * ps < ctx.max_total_len:
+                raise K.KernelError("attention: the block tables are narrower than the longest request")
+            n = K.decode_splits(nd, nh, nkv, self._span(ctx.max_total_len), dev, d)
+            if nd * n > records:
+                raise K.KernelError("attention: the parts of the keys do not fit the program's arena")
+            return n
+
+        def launch_shape(ctx: StepContext) -> int:
+            nd = ctx.num_decode
+            if ctx.num_seqs == nd:
+                return 0
+            return K.prefill_launch_shape(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:], window, dev)
+        return (program.scalar(("attention: parts of the keys", nh, nkv, g, ps), parts_of_the_keys),
+                program.scalar(("attention: launch shape", nh, nkv, d, window), launch_shape))
+
+    def emit_attend(self, program, view: CacheView, q, q_stride: int, when, out=None):
+        """The launches of :meth:`attend` alone, for queries ``q`` (rows of ``q_stride`` values, the heads first) that
+        are rotated already and whose keys and values are in their pages: the kernel for single tokens on the first
+        rows and the one for portions of prompts on the rest, or the plain kernel on all rows.  Returns the buffer
+        [N, nh d] of the attended rows."""
+        from ..engine.program import STREAM, Guard
+        nh, nkv, d, window, rt = self.nh, self.nkv, self.d, self.mask, self.rt
+        k, v, g = view.k_pages, view.v_pages, view.group
+        ps, num_pages = int(k.shape[2]), int(k.shape[0])
+        T, act, scale = program.T, program.act_code, float(self.scale)
+        program.keep(k, v)
+        bt, bt_cols = program.block_table(g), program.bt_cols(g)
+        if out is None:
+            out = program.buffer("attention.out", T * nh * d * program.act_bytes)
+        if not (self.use_mfma and ps % 4 == 0):
+            program.op("core", "ia_attention_generic",
+                       [q, q_stride, k, v, out, nh * d, act, program.token_seq, program.positions, bt, bt_cols, program.N,
+                        nh, nkv, d, ps, num_pages, scale, window, STREAM], when)
+            return out
+        lib = K._attn(d)
+        records = T + 1024
+        part_o = program.buffer("attention.part_o", records * nh * d * 4)
+        part_ml = program.buffer("attention.part_ml", records * nh * 2 * 4)
+        splits, shape = self._attend_scalars(program, g, ps, records)
+        tiles, num_tiles = program.row_tiles(K.PREFILL_TILE_ROWS)
+        program.op(lib, "ia_attn_decode",
+                   [q, q_stride, k, v, out, nh * d, part_o, part_ml, program.positions, bt, bt_cols, program.ND, nh,
+                    nkv, ps, num_pages, scale, window, splits, STREAM], when & Guard.between(program.ND, 1))
+        program.op(lib, "ia_attn_prefill",
+                   [q, q_stride, k, v, out, nh * d, program.seq_starts, program.seq_ctx, bt, bt_cols, tiles, num_tiles,
+                    nh, nkv, ps, num_pages, scale, window, shape, STREAM], when & Guard.between(program.NP, 1))
+        return out
+
+    def _span(self, max_len: int) -> int:
+        """The most keys a query can see, given the longest request: what the decode kernel's choice of parts
+        goes by (under chunks a query never sees more than its chunk)."""
+        return min(max_len, self.chunk) if self.chunk else max_len
 
     def attend(self, qkv: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: CacheView) -> None:
         nh, nkv, d = self.nh, self.nkv, self.d
         bt = ctx.block_tables[cache.group]
         if not self.use_mfma or cache.k_pages.shape[2] % 4:
             K.attention_generic(qkv, cache.k_pages, cache.v_pages, out, ctx.token_seq, ctx.positions, bt, nh, nkv, d,
-                                self.scale, self.window)
+                                self.scale, self.mask)
             return
         nd = ctx.num_decode
         if nd > 0:
             K.attention_decode(qkv[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.positions[:nd], bt[:nd], nh, nkv,
-                               d, self.scale, self.window, ctx.max_total_len)
+                               d, self.scale, self.mask, self._span(ctx.max_total_len))
         if ctx.num_seqs > nd:
-            key = ("prefill_launch_shape", nh, nkv, d, self.window)
+            key = ("prefill_launch_shape", nh, nkv, d, self.mask)
             hpw = ctx.extras.get(key)
             if hpw is None:             # once per step for all layers of this shape
                 hpw = ctx.extras[key] = K.prefill_launch_shape(nh, nkv, d, ctx.q_lens[nd:], ctx.ctx_lens[nd:],
-                                                               self.window, qkv.device)
+                                                               self.mask, qkv.device)
             tiles, num_tiles = ctx.row_tiles(K.PREFILL_TILE_ROWS)
             K.attention_prefill(qkv, cache.k_pages, cache.v_pages, out, ctx.seq_starts, ctx.seq_ctx, bt,
-                                tiles, num_tiles, nh, nkv, d, self.scale, self.window, hpw)
+                                tiles, num_tiles, nh, nkv, d, self.scale, self.mask, hpw)
 
 
 register_part("mixer", "attention", Attention)

@@ -1,7 +1,7 @@
 """Arrangements of a layer's parts around the fp32 residual stream.
 
 ``prenorm``: h' = h + mixer(norm1(h)); h'' = h' + feed_forward(norm2(h'))
-(infernum-llama/src/graph_builder.rs:453-507).  Each add is carried as a pending
+(infernum-llama/src/graph_builder.rs:453-507); without a feed-forward the layer ends after its first sublayer.  Each add is carried as a pending
 delta into the next norm, which adds and normalises in one pass over the row
 (the reference's add_rmsnorm fusion, infernum/src/graph/optimizer.rs:105-174,
 there limited to adds with one consumer).
@@ -23,21 +23,33 @@ from .base import Block, CacheView, StepContext, register_part
 
 
 class PreNormBlock(Block):
+    """The feed-forward (with its norm) may be absent: the layer is then its first sublayer alone.  An extra part
+    ``stream_in`` (category "stream_in") rewrites the residual stream before the layer's first norm."""
     graph_safe = True
+
     def forward(self, h: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
                 cache: CacheView) -> torch.Tensor:
+        stream_in = self.extra.get("stream_in")
+        if stream_in is not None:
+            stream_in.forward(h, pending, ctx)
+            pending = None
         n = self.mixer_norm.forward(h, pending)
         a = self.mixer.forward(n, ctx, cache)
+        if self.feed_forward is None:
+            return a
         n = self.feed_forward_norm.forward(h, a)
         return self.feed_forward.forward(n, ctx)
 
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not PreNormBlock.forward:
             return super().native(program, view)
+        if self.extra.get("stream_in") is not None:
+            self.extra["stream_in"].native(program, None)
         self.mixer_norm.native(program, None)
         self.mixer.native(program, view)
-        self.feed_forward_norm.native(program, None)
-        self.feed_forward.native(program, None)
+        if self.feed_forward is not None:
+            self.feed_forward_norm.native(program, None)
+            self.feed_forward.native(program, None)
 
 
 class BranchNormBlock(Block):

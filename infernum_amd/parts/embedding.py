@@ -18,13 +18,19 @@ from .base import Embedding, Head, Runtime, StepContext, WeightSpec, register_pa
 from .linear import emit_linear, linear
 
 
+EMBEDDING_OUTPUT = "embedding.out"
+
+
 class TokenEmbedding(Embedding):
     graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, init_std: float = 0.02, scale: float = 1.0,
-                 name: str = "weight"):
+                 name: str = "weight", keep_output: bool = False):
         """``scale`` multiplies the looked-up row in fp32 (the table itself stays as stored: a head tied to it
-        reads it unscaled); ``name`` is the table's local tensor name."""
+        reads it unscaled); ``name`` is the table's local tensor name.  ``keep_output``: the rows as they leave
+        here stay available to later parts of the step, rounded to the compute dtype (``EMBEDDING_OUTPUT`` in
+        ``ctx.extras``, or the program's buffer of that name)."""
         super().__init__(rt)
+        self.keep_output = bool(keep_output)
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.init_std = init_std
         self.scale, self.name = float(scale), str(name)
@@ -38,7 +44,10 @@ class TokenEmbedding(Embedding):
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         h = torch.empty((ctx.num_tokens, self.hidden_size), dtype=torch.float32, device=self.table.device)
-        return K.embed(self.table, ctx.token_ids, h, self.scale)
+        K.embed(self.table, ctx.token_ids, h, self.scale)
+        if self.keep_output:
+            ctx.extras[EMBEDDING_OUTPUT] = K.cast(h, self.rt.dtype)
+        return h
 
     def native(self, program, view=None) -> None:
         if type(self).forward is not TokenEmbedding.forward:
@@ -46,35 +55,48 @@ class TokenEmbedding(Embedding):
         from ..engine.program import STREAM
         program.op("core", "ia_embed", [self.table, K.DTYPE_CODE[self.table.dtype], program.token_ids, program.h,
                                         program.N, self.hidden_size, self.vocab_size, float(self.scale), STREAM])
+        if self.keep_output:
+            kept = program.buffer(EMBEDDING_OUTPUT, program.T * self.hidden_size * program.act_bytes)
+            program.op("core", "ia_cast", [program.h, K.DTYPE_CODE[torch.float32], kept, program.act_code,
+                                           program.N * self.hidden_size, STREAM])
         program.pending = None
 
 
 class LinearHead(Head):
     graph_safe = True
     def __init__(self, rt: Runtime, vocab_size: int, hidden_size: int, fallback: Optional[str] = None,
-                 tied: bool = False, init_std: float = 0.02):
+                 tied: bool = False, init_std: float = 0.02, name: str = "weight", softcap: Optional[float] = None):
+        """``softcap`` c: the logits become c tanh(logits / c).  ``name``: the matrix's local tensor name."""
         super().__init__(rt)
+        self.name = str(name)
+        self.softcap = float(softcap) if softcap else 0.0
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.fallback, self.tied, self.init_std = fallback, bool(tied), init_std
         self.weight: Optional[torch.Tensor] = None
 
     def weights(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std),
+        return {self.name: WeightSpec((self.vocab_size, self.hidden_size), ("normal", self.init_std),
                                      fallback=self.fallback, write_when_random=not self.tied)}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         # no second copy laid out for the weight-streaming kernel: since that kernel's tiles of rows walk K from
         # starts of their own, the file's layout serves the head as well (128,256 x 4,096 on an MI355X: 187.1 against
         # 187.6 us at 8 rows, 190.0 against 189.0 at 16), and a copy would be another gigabyte
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.name]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
+        logits = linear(x, self.weight, out_dtype=torch.float32, kernels=self.rt.kernels)
+        if self.softcap and logits.shape[0]:
+            logits = K.softcap(logits if logits.is_contiguous() else logits.contiguous(), self.softcap)
+        return logits
 
     def native(self, program, view=None) -> None:
         if type(self).forward is not LinearHead.forward:
             return super().native(program, view)
         emit_linear(program, program.x, program.R, self.weight, torch.float32, None, False, program.logits, "head")
+        if self.softcap:
+            from ..engine.program import STREAM
+            program.op("core", "ia_softcap", [program.logits, program.R, self.vocab_size, float(self.softcap), STREAM])
 
 
 register_part("embedding", "token", TokenEmbedding)

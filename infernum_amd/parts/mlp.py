@@ -19,25 +19,25 @@ from .linear import emit_linear, linear, prepare_weights
 
 class SwiGLUFeedForward(FeedForward):
     graph_safe = True
-    def __init__(self, rt: Runtime, hidden_size: int, intermediate_size: int, init_std: float = 0.02):
+    def __init__(self, rt: Runtime, hidden_size: int, intermediate_size: int, init_std: float = 0.02,
+                 names: Sequence[str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        """``names``: the local tensor names of the gate, up and down matrices."""
         super().__init__(rt)
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
-        self.init_std = init_std
+        self.init_std, self.names = init_std, tuple(names)
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
 
     def weights(self) -> Dict[str, WeightSpec]:
         H, I = self.hidden_size, self.intermediate_size
         init = ("normal", self.init_std)
-        return {
-            "gate_proj.weight": WeightSpec((I, H), init),
-            "up_proj.weight": WeightSpec((I, H), init),
-            "down_proj.weight": WeightSpec((H, I), init),
-        }
+        gate, up, down = self.names
+        return {gate: WeightSpec((I, H), init), up: WeightSpec((I, H), init), down: WeightSpec((H, I), init)}
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"].contiguous()
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+        self.w_down = tensors[down].contiguous()
         prepare_weights(self.rt, [(self.w_gate_up, "swiglu", False), (self.w_down, None, True)])
 
     def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None):

@@ -13,6 +13,13 @@ context n, L < n/high keeps f, L > n/low gives f/factor, and between them
 f' = (1-r) f/factor + r f with r = (n/L - low) / (high - low).  There is no
 magnitude correction.
 
+``yarn`` scaling (keys ``factor``, ``original``, ``fast``, ``slow``) blends by the pair's index instead of its
+wavelength: with dim(t) = rot ln(original / (2 pi t)) / (2 ln theta), the index at which a pair makes t turns over the
+original context, lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), rot - 1) and
+r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * r_i + f_i (1 - r_i); sine and cosine
+are both multiplied by ``magnitude`` = 0.1 ln(factor) + 1 (the reference's YaRN, infernum/src/rope.rs:91-120, has the
+same bands and correction).  ``pairing`` "neighbours" pairs value 2i with value 2i + 1 in place of i with i + rot/2.
+
 Frequencies are formed and kept in float64; the rotation kernel forms the angle
 position * frequency in float64 too and brings it into [-pi, pi] before it takes
 the fp32 sine and cosine, so that the angle is as good at position 100,000 as at
@@ -39,6 +46,9 @@ def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Ma
         f = float(theta) ** (-2.0 * i / rotary_dim)
         if scaling is not None:
             kind = scaling.get("rope_type")
+            if kind == "yarn":
+                freqs.append(f)
+                continue
             if kind != "llama3":
                 raise ValueError(f"rope scaling of type {kind!r} is not supported")
             factor = float(scaling["factor"])
@@ -54,7 +64,24 @@ def rope_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Ma
                 r = (n / wavelen - low) / (high - low)
                 f = (1.0 - r) * f / factor + r * f
         freqs.append(f)
+    if scaling is not None and scaling.get("rope_type") == "yarn":
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+
+        def index_of_turns(turns: float) -> float:
+            return rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(theta)))
+        lo = max(math.floor(index_of_turns(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(index_of_turns(float(scaling["slow"]))), rotary_dim - 1)
+        for i in range(half):
+            r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            freqs[i] = freqs[i] / factor * r + freqs[i] * (1.0 - r)
     return torch.tensor(freqs, dtype=torch.float64)
+
+
+def rope_magnitude(scaling: Optional[Mapping[str, Any]]) -> float:
+    """The factor on sine and cosine: 0.1 ln(factor) + 1 under ``yarn`` scaling, 1 otherwise."""
+    if scaling is not None and scaling.get("rope_type") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 class RotaryEmbedding(PositionEncoding):
@@ -62,13 +89,25 @@ class RotaryEmbedding(PositionEncoding):
     graph_safe = True
 
     def __init__(self, rt: Runtime, head_dim: int, theta: float, scaling: Optional[Mapping[str, Any]] = None,
-                 rotary_dim: Optional[int] = None):
+                 rotary_dim: Optional[int] = None, pairing: str = "half"):
         super().__init__(rt)
         self.head_dim = int(head_dim)
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
         if self.rotary_dim > self.head_dim:
             raise ValueError("rotary_dim larger than the head size")
+        if pairing not in ("half", "neighbours"):
+            raise ValueError(f"pairing {pairing!r}: 'half' or 'neighbours'")
+        self.pairing = pairing
+        self.magnitude = rope_magnitude(scaling)
         self.inv_freq = rope_inverse_frequencies(self.rotary_dim, theta, scaling).to(rt.device)
+
+    def head_permutation(self) -> Optional[torch.Tensor]:
+        """For kernels that pair value i with value i + rot/2: the order of a head's values that makes those pairs
+        the neighbours' (kernels that take a pairing need none)."""
+        if self.pairing == "half":
+            return None
+        r = self.rotary_dim
+        return torch.tensor(list(range(0, r, 2)) + list(range(1, r, 2)) + list(range(r, self.head_dim)), dtype=torch.int64)
 
 
 class NoPositionEncoding(PositionEncoding):
@@ -79,6 +118,7 @@ class NoPositionEncoding(PositionEncoding):
         super().__init__(rt)
         self.inv_freq = None
         self.rotary_dim = 0
+        self.pairing, self.magnitude = "half", 1.0
 
 
 register_part("position", "rope", RotaryEmbedding)
