@@ -48,7 +48,7 @@ class ConvAttentionConfig:
     vdim: int
     conv: int                   # taps of the convolution on queries and keys
     scale: float
-    rot_base: float
+    rot_base: Optional[float]   # None: the file has no 'rot' at all
     rot_dims: int               # how many of a head's first values are rotated
     rot_scaling: Optional[RotScaling]
     chunk: Optional[int]        # a query sees the keys of its own chunk of so many positions; None: all earlier keys
@@ -61,7 +61,7 @@ class ConvAttentionConfig:
             heads=r.integer("heads", minimum=1), kv_heads=r.integer("kv_heads", minimum=1),
             dim=r.integer("dim", minimum=1), vdim=r.integer("vdim", minimum=1), conv=r.integer("conv", minimum=1),
             scale=r.number("scale", positive=True),
-            rot_base=rot.number("base", positive=True) if rot is not None else 10000.0,
+            rot_base=rot.number("base", positive=True) if rot is not None else None,
             rot_dims=rot.integer("dims", minimum=0) if rot is not None else 0,
             rot_scaling=RotScaling(sc.number("factor", positive=True), sc.number("original", positive=True),
                                    sc.number("fast", positive=True), sc.number("slow", positive=True)) if sc is not None else None,
@@ -76,7 +76,9 @@ class ConvAttentionConfig:
 
     def to_dict(self) -> dict:
         out = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv,
-               "scale": self.scale, "rot": {"base": self.rot_base, "dims": self.rot_dims}}
+               "scale": self.scale}
+        if self.rot_base is not None:
+            out["rot"] = {"base": self.rot_base, "dims": self.rot_dims}
         if self.rot_scaling is not None:
             out["rot"]["scaling"] = self.rot_scaling.to_dict()
         if self.chunk is not None:

@@ -46,14 +46,11 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     T, C = u.shape
     taps = w.shape[1]
     y = torch.zeros_like(u)
-    for t in range(T):
-        for j in range(taps):
-            s = t - (taps - 1) + j
-            if s >= 0:
-                y[t] += w[:, j] * u[s]
-        if bias is not None:
-            y[t] += bias
-    return y
+    for j in range(taps):
+        lag = taps - 1 - j                      # tap j meets the input lag tokens back
+        if lag < T:
+            y[lag:] += w[:, j] * u[:T - lag]
+    return y if bias is None else y + bias
 
 
 def rotary_frequencies(rot: dict) -> (torch.Tensor, float):
@@ -116,8 +113,9 @@ def conv_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: fl
     q = _r(causal_conv(q, w["q.conv"]), round_to).view(T, H, d)
     k = _r(causal_conv(k, w["k.conv"]), round_to).view(T, G, d)
     v = k
-    q = rotate_neighbours(weighted_norm(q, w["q.norm"], eps), pos, m["rot"])
-    k = rotate_neighbours(weighted_norm(k, w["k.norm"], eps), pos, m["rot"])
+    rot = m.get("rot") or {"dims": 0, "base": 10000.0}
+    q = rotate_neighbours(weighted_norm(q, w["q.norm"], eps), pos, rot)
+    k = rotate_neighbours(weighted_norm(k, w["k.norm"], eps), pos, rot)
     q, k = _r(q, round_to), _r(k, round_to)
     mask = chunk_visible(T, (m.get("mask") or {}).get("size"))
     out = torch.zeros(T, H, d, dtype=h.dtype)
@@ -147,12 +145,12 @@ def mamba2(h: torch.Tensor, w: Dict[str, torch.Tensor], m: dict, eps: float,
     dt = softplus(dt + w["dt_bias"])                                     # [T, nh]
     decay = torch.exp(-torch.exp(w["A_log"])[None, :] * dt)              # [T, nh]
     y = torch.zeros(T, nh, P, dtype=h.dtype)
-    for hd in range(nh):
-        g = hd // (nh // G)
-        S = torch.zeros(N, P, dtype=h.dtype)
-        for t in range(T):
-            S = decay[t, hd] * S + dt[t, hd] * torch.outer(B[t, g], x[t, hd])
-            y[t, hd] = S.t() @ C[t, g] + w["D"][hd] * x[t, hd]
+    per = nh // G
+    S = torch.zeros(nh, N, P, dtype=h.dtype)                             # all heads side by side, token after token
+    for t in range(T):
+        Bh, Ch = B[t].repeat_interleave(per, dim=0), C[t].repeat_interleave(per, dim=0)      # [nh, N]
+        S = decay[t][:, None, None] * S + dt[t][:, None, None] * Bh[:, :, None] * x[t][:, None, :]
+        y[t] = (S * Ch[:, :, None]).sum(dim=1) + w["D"][:, None] * x[t]
     y = y.reshape(T, inner) * silu(z)
     y = unit_rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * w["norm"]
     return _r(_r(y, round_to) @ w["o"].t(), round_to)
