@@ -479,18 +479,74 @@ def nesilorn_active_params(size: dict) -> int:
     return n * mixer + (n - n // 2) * dense + (n // 2) * routed + size["vocab"] * W
 
 
+# ---- the Rogizen design beside the Llama decoder at equal sizes -------------------------------------------------
+# Eight layers of one width: three state-space layers (inner size twice the width, heads of 64, a state of 128, eight
+# groups), then an attention layer whose queries and keys are convolved (heads of 128 over 4 key/value heads, chunks
+# of 1,024, half of a head rotated with scaled frequencies), twice; every layer with the gated feed-forward of the
+# Llama twin, which has the same width, layers, vocabulary, heads and feed-forward.  The eight layers are one pass of
+# a loop, so the matrix over stream and embedding is in the step.
+ROGIZEN_SIZES = {
+    "2k": dict(width=2048, layers=8, vocab=32000, ff=5504, heads=16, kv_heads=4, dim=128, chunk=1024, taps=4,
+               ssm_heads=64, ssm_vdim=64, state=128, groups=8, norm_groups=8),
+    "4k": dict(width=4096, layers=8, vocab=32000, ff=9600, heads=32, kv_heads=8, dim=128, chunk=2048, taps=4,
+               ssm_heads=128, ssm_vdim=64, state=128, groups=8, norm_groups=8),
+}
+
+
+def rogizen_configs(size: dict):
+    from infernum_amd.config import LlamaConfig
+    from infernum_amd.config.rogizen import RogizenConfig
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+                 "conv": size["taps"], "scale": size["dim"] ** -0.5, "mask": {"size": size["chunk"]},
+                 "rot": {"base": 10000.0, "dims": size["dim"] // 2,
+                         "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    ssm = {"heads": size["ssm_heads"], "vdim": size["ssm_vdim"], "state": size["state"], "groups": size["groups"],
+           "norm_groups": size["norm_groups"], "conv": size["taps"]}
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    rog = RogizenConfig.from_dict({
+        "architecture": "Rogizen", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+        "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": {"start": 0, "stop": size["layers"], "times": 1},
+        "layers": [{"type": "attention", "mixer": attention, "mlp": mlp} if i % 4 == 3 else
+                   {"type": "mamba2", "mixer": ssm, "mlp": mlp} for i in range(size["layers"])]})
+    llama = LlamaConfig.from_dict(dict(
+        model_type="llama", num_hidden_layers=size["layers"], hidden_size=size["width"],
+        num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], intermediate_size=size["ff"],
+        vocab_size=size["vocab"], rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+        max_position_embeddings=8192))
+    return rog, llama
+
+
+def rogizen_active_params(size: dict) -> int:
+    """Weights that a token multiplies with in the Rogizen model of these sizes (the head included)."""
+    W, n = size["width"], size["layers"]
+    inner = size["ssm_heads"] * size["ssm_vdim"]
+    ssm = W * (2 * inner + 2 * size["groups"] * size["state"] + size["ssm_heads"]) + inner * W
+    attention = W * (size["heads"] + size["kv_heads"]) * size["dim"] + size["heads"] * size["dim"] * W
+    return (n // 4) * attention + (n - n // 4) * ssm + n * 3 * W * size["ff"] + 2 * W * W + size["vocab"] * W
+
+
 def nesilorn_bench(a) -> int:
-    """Prefill of 2,048 tokens and decode steps at batch 8 and 64 of the Nesilorn design and of the Llama decoder
-    at equal sizes, random weights, through the same engine and generation loop; one JSON line of its own."""
+    batches = [int(b) for b in a.nesilorn_batches.split(",") if b]
+    return beside_llama_bench(a, "Nesilorn", [(n, NESILORN_SIZES[n]) for n in a.nesilorn.split(",")], nesilorn_configs,
+                              nesilorn_active_params, batches)
+
+
+def rogizen_bench(a) -> int:
+    batches = [int(b) for b in a.rogizen_batches.split(",") if b]
+    return beside_llama_bench(a, "Rogizen", [(n, ROGIZEN_SIZES[n]) for n in a.rogizen.split(",")], rogizen_configs,
+                              rogizen_active_params, batches)
+
+
+def beside_llama_bench(a, design, sizes, configs, active_params, batches) -> int:
+    """Prefill of 2,048 tokens and decode steps at batch 8 and 64 of a design and of the Llama decoder at equal
+    sizes, random weights, through the same engine and generation loop; one JSON line of its own."""
     import torch
     from infernum_amd import CacheConfig, Engine
     from infernum_amd.engine import StepEntry
-    out = {"metric": "Nesilorn beside Llama at equal sizes", "dtype": "bf16", "data": "synthetic", "sizes": {}}
-    batches = [int(b) for b in a.nesilorn_batches.split(",") if b]
-    for name in a.nesilorn.split(","):
-        size = NESILORN_SIZES[name]
+    out = {"metric": f"{design} beside Llama at equal sizes", "dtype": "bf16", "data": "synthetic", "sizes": {}}
+    for name, size in sizes:
         rec = {"config": {k: v for k, v in size.items()}}
-        for label, cfg in zip(("nesilorn", "llama"), nesilorn_configs(size)):
+        for label, cfg in zip((design.lower(), "llama"), configs(size)):
             max_batch = max(batches)
             tokens = max(max_batch * (PROMPT_LEN + a.steps + a.warmup + prefill_steps(max_batch, PROMPT_LEN) + 2 * PAGE_SIZE),
                          PREFILL_TOKENS + PAGE_SIZE)
@@ -518,8 +574,8 @@ def nesilorn_bench(a) -> int:
                 dt, _ = time_decode(engine, b, steps, max(4, min(a.warmup, 8)), PROMPT_LEN)
                 r[f"decode_b{b}_tok_per_s"] = round(b * steps / dt, 1)
                 r[f"decode_b{b}_ms_per_step"] = round(dt / steps * 1e3, 3)
-            if label == "nesilorn":
-                active = nesilorn_active_params(size)
+            if label != "llama":
+                active = active_params(size)
             else:
                 per_layers, head = matmul_params(cfg)
                 active = per_layers + head
@@ -571,6 +627,11 @@ def main() -> int:
                     help="the Nesilorn design (latent attention, routed experts) beside the Llama decoder at equal sizes "
                          "instead: prefill and decode of each (a JSON line of its own); sizes: 2k, 4k or both with a comma")
     ap.add_argument("--nesilorn-batches", default="8,64", help="decode batches of --nesilorn")
+    ap.add_argument("--rogizen", default="", metavar="SIZES",
+                    help="the Rogizen design (state-space layers, attention with convolved queries and keys) beside the "
+                         "Llama decoder at equal sizes instead: prefill and decode of each (a JSON line of its own); "
+                         "sizes: 2k, 4k or both with a comma")
+    ap.add_argument("--rogizen-batches", default="8,64", help="decode batches of --rogizen")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for --gpus {a.gpus})")
@@ -578,6 +639,8 @@ def main() -> int:
 
     if a.nesilorn:
         return nesilorn_bench(a)
+    if a.rogizen:
+        return rogizen_bench(a)
     if a.decode_kernels:
         return decode_kernels_alone(a)
     if a.serve:
