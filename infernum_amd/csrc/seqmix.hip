@@ -9,7 +9,8 @@
 //                          cosine, the keys to their pages, and as values either the value heads of the row or the
 //                          key heads as they came in
 //   ia_ssd_scan            the selective state-space recurrence  S <- a S + dt B x^T,  y = S^T C + D x  per head,
-//                          the state [N, P] of every request in its slot (fp32)
+//                          the state [N, P] of every request in its slot (fp32), token after token
+//   ia_ssd_chunked         the same recurrence as matrix products over chunks of 64 tokens, for portions of prompts
 //   ia_gated_group_norm    y * silu(z), then an RMS norm in equal parts of the row, times a weight
 //   ia_concat_cast         rows [cast(a) | b]: the operand of a product over two streams side by side
 //   ia_stream_add         the fp32 stream += a tensor or the partial sums of a split product
@@ -315,6 +316,203 @@ extern "C" int ia_ssd_scan(const void* xbc, int code, int xbc_stride, const void
   return IA_OK;
 }
 
+// ------------------------------------------------------------------------------------------ the recurrence, in chunks
+// The same recurrence for steps that bring portions of prompts, as matrix products over chunks of 64 tokens.  With
+// a_i = -exp(a_log) dt_i and c_i = a_1 + ... + a_i inside a chunk that starts from the state S0:
+//
+//   y_i = exp(c_i) C_i^T S0 + sum_{j <= i} exp(c_i - c_j) dt_j (C_i . B_j) x_j + D x_i
+//   S   = exp(c_L) S0 + sum_j exp(c_L - c_j) dt_j B_j x_j^T
+//
+// One workgroup of four waves per (request, head, 16 of the head's P values) walks the request's chunks in order.
+// C B^T is a bf16 product (B and C are bf16 values as stored, so nothing is rounded) with fp32 sums; everything that
+// carries a decay, a step size or the state is fp32 on v_mfma_f32_16x16x4_f32: every exponent is at most zero.  The
+// state of the slice lives in LDS between chunks.  Rows past a request's last token are zero with dt = 0, which
+// leaves sums and state as they are.
+typedef __bf16 sm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
+
+#define SSD_L 64          // tokens of a chunk
+#define SSD_PW 16         // values of a head that a workgroup owns
+#define SSD_GS 68         // row stride of the chunk's [L, L] matrix in LDS, floats
+#define SSD_XS 20         // row stride of x and of the state in LDS, floats
+
+__global__ __launch_bounds__(256) void ssd_chunk_kernel(
+    const bf16_t* __restrict__ xbc, int xbc_stride, const bf16_t* __restrict__ dt_raw, int dt_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ skip,
+    float* __restrict__ state, long state_stride, float* __restrict__ y, const int* __restrict__ seq_starts,
+    const int* __restrict__ state_slots, int nh, int P, int Ns, int G, int NP) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ssd_lds[];
+  const int BS = NP + 8;                                   // row stride of B and C in LDS, bf16 values
+  uint16_t* Bs = (uint16_t*)ssd_lds;                       // [L][BS]
+  uint16_t* Cs = Bs + SSD_L * BS;                          // [L][BS]
+  float* Gs = (float*)(Cs + SSD_L * BS);                   // [L][GS]
+  float* Xs = Gs + SSD_L * SSD_GS;                         // [L][XS]
+  float* Ss = Xs + SSD_L * SSD_XS;                         // [Ns][XS]
+  float* cum = Ss + (size_t)Ns * SSD_XS;                   // [L]
+  float* dts = cum + SSD_L;                                // [L]
+  const int slices = P / SSD_PW;
+  const int hd = blockIdx.x / slices, ps = blockIdx.x - hd * slices;
+  const int s = blockIdx.y;
+  const int first = seq_starts[s], q = seq_starts[s + 1] - first;
+  if (q <= 0) return;
+  const int g = hd / (nh / G);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l15 = lane & 15, kk = lane >> 4;
+  float* S = state + (size_t)state_slots[s] * state_stride + (size_t)hd * Ns * P + (size_t)ps * SSD_PW;
+  const float A = -expf(a_log[hd]);
+  const float bias = dt_bias[hd], D = skip[hd];
+  const size_t x_col = (size_t)hd * P + (size_t)ps * SSD_PW;
+  const size_t b_col = (size_t)nh * P + (size_t)g * Ns, c_col = b_col + (size_t)G * Ns;
+  const int yw = nh * P;
+  // the state of the slice, and zeros in the columns of B and C past the state's size
+  for (int i = tid; i < Ns * SSD_PW; i += 256) Ss[(i >> 4) * SSD_XS + (i & 15)] = S[(size_t)(i >> 4) * P + (i & 15)];
+  if (NP > Ns)
+    for (int i = tid; i < SSD_L * (NP - Ns); i += 256) {
+      const int r = i / (NP - Ns), c = Ns + i % (NP - Ns);
+      Bs[r * BS + c] = 0;
+      Cs[r * BS + c] = 0;
+    }
+  const int vec_row = Ns >> 3;                             // 16-byte pieces of a row of B or C
+  for (int c0 = 0; c0 < q; c0 += SSD_L) {
+    const int Lc = q - c0 < SSD_L ? q - c0 : SSD_L;
+    const size_t row0 = (size_t)(first + c0);
+    __syncthreads();                                       // the chunk before is done with B, C, x and the sums
+    // ---- B, C, x of the chunk; step sizes and the running sum of a
+    for (int i = tid; i < SSD_L * vec_row; i += 256) {
+      const int r = i / vec_row, v = i - r * vec_row;
+      uint4 bv = make_uint4(0, 0, 0, 0), cv = bv;
+      if (r < Lc) {
+        bv = *(const uint4*)(xbc + (row0 + r) * xbc_stride + b_col + 8 * v);
+        cv = *(const uint4*)(xbc + (row0 + r) * xbc_stride + c_col + 8 * v);
+      }
+      *(uint4*)(Bs + r * BS + 8 * v) = bv;
+      *(uint4*)(Cs + r * BS + 8 * v) = cv;
+    }
+    for (int i = tid; i < SSD_L * SSD_PW; i += 256) {
+      const int r = i >> 4, c = i & 15;
+      Xs[r * SSD_XS + c] = r < Lc ? to_float(xbc[(row0 + r) * xbc_stride + x_col + c]) : 0.f;
+    }
+    if (wave == 0) {
+      float dt = 0.f;
+      if (lane < Lc) {
+        const float z = to_float(dt_raw[(row0 + lane) * dt_stride + hd]) + bias;
+        dt = z > 20.f ? z : log1pf(expf(z));
+      }
+      float c = A * dt;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(c, o, 64);
+        if (lane >= o) c += up;
+      }
+      cum[lane] = c;
+      dts[lane] = dt;
+    }
+    __syncthreads();
+    // ---- G[i][j] = (C_i . B_j) exp(c_i - c_j) dt_j for j <= i: wave w makes rows 16 w .. 16 w + 15
+    for (int jt = 0; jt <= wave; ++jt) {
+      sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      const uint16_t* cp = Cs + (16 * wave + l15) * BS + 8 * kk;
+      const uint16_t* bp = Bs + (16 * jt + l15) * BS + 8 * kk;
+      for (int k0 = 0; k0 < NP; k0 += 32) {
+        const sm_bf16x8 a = *(const sm_bf16x8*)(cp + k0);
+        const sm_bf16x8 b = *(const sm_bf16x8*)(bp + k0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+      }
+      const int j = 16 * jt + l15;
+      const float cj = cum[j], dj = dts[j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * wave + 4 * kk + r;
+        Gs[i * SSD_GS + j] = j <= i ? acc[r] * expf(cum[i] - cj) * dj : 0.f;
+      }
+    }
+    __syncthreads();
+    // ---- y rows 16 w .. 16 w + 15 of the chunk: G x + exp(c_i) C S0 + D x
+    {
+      sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      const int i = 16 * wave + l15;                       // the row this lane feeds
+      for (int jb = 0; jb <= wave; ++jb) {
+        const sm_f32x4 a = *(const sm_f32x4*)(Gs + i * SSD_GS + 16 * jb + 4 * kk);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], Xs[(16 * jb + 4 * kk + r) * SSD_XS + l15], acc, 0, 0, 0);
+      }
+      const float ei = expf(cum[i]);
+      for (int nb = 0; nb < Ns; nb += 16) {
+        const uint2 cw = *(const uint2*)(Cs + i * BS + nb + 4 * kk);
+        const float a0 = __uint_as_float(cw.x << 16) * ei, a1 = __uint_as_float(cw.x & 0xffff0000u) * ei;
+        const float a2 = __uint_as_float(cw.y << 16) * ei, a3 = __uint_as_float(cw.y & 0xffff0000u) * ei;
+        const float* sp = Ss + (nb + 4 * kk) * SSD_XS + l15;
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, sp[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, sp[SSD_XS], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a2, sp[2 * SSD_XS], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a3, sp[3 * SSD_XS], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int io = 16 * wave + 4 * kk + r;
+        if (io < Lc)
+          y[(row0 + io) * yw + x_col + l15] = __builtin_fmaf(D, Xs[io * SSD_XS + l15], acc[r]);
+      }
+    }
+    __syncthreads();                                       // every wave has read S0
+    // ---- the state after the chunk: tiles of 16 state rows, wave w takes tiles w, w + 4, ...
+    {
+      const float clast = cum[SSD_L - 1];
+      const float keep = expf(clast);
+      for (int nt = wave; 16 * nt < Ns; nt += 4) {
+        sm_f32x4 acc;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = keep * Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15];
+        for (int jb = 0; jb < SSD_L; jb += 16) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = jb + 4 * kk + r;
+            const float wj = expf(clast - cum[j]) * dts[j];
+            const float a = __uint_as_float((uint32_t)Bs[j * BS + 16 * nt + l15] << 16) * wj;
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Xs[j * SSD_XS + l15], acc, 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15] = acc[r];
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < Ns * SSD_PW; i += 256) S[(size_t)(i >> 4) * P + (i & 15)] = Ss[(i >> 4) * SSD_XS + (i & 15)];
+}
+
+// Whether ia_ssd_chunked takes these sizes (otherwise ia_ssd_scan does the step).
+extern "C" int ia_ssd_chunked_takes(int nh, int P, int Ns, int G, int xbc_stride) {
+  return nh > 0 && G > 0 && nh % G == 0 && P % SSD_PW == 0 && Ns % 16 == 0 && Ns >= 16 && Ns <= 256 && xbc_stride % 8 == 0;
+}
+
+extern "C" int ia_ssd_chunked(const void* xbc, int code, int xbc_stride, const void* dt_raw, int dt_stride,
+                              const float* dt_bias, const float* a_log, const float* skip, float* state,
+                              long state_stride, float* y, const int* seq_starts, const int* state_slots, int B, int nh,
+                              int P, int Ns, int G, hipStream_t stream) {
+  if (B == 0) return IA_OK;
+  if (!xbc || !dt_raw || !dt_bias || !a_log || !skip || !state || !y || !seq_starts || !state_slots || B < 0 ||
+      B > 65535 || nh <= 0 || P <= 0 || Ns <= 0 || G <= 0 || nh % G || xbc_stride < nh * P + 2 * G * Ns ||
+      dt_stride < nh || state_stride < (long)nh * Ns * P || ((uintptr_t)xbc & 15))
+    return IA_ERR_BAD_ARG;
+  if (code != IA_BF16 || !ia_ssd_chunked_takes(nh, P, Ns, G, xbc_stride)) return IA_ERR_UNSUPPORTED;
+  const int NP = (Ns + 31) / 32 * 32;
+  const size_t lds = 2 * (size_t)SSD_L * (NP + 8) * 2 + sizeof(float) * ((size_t)SSD_L * SSD_GS + (size_t)SSD_L * SSD_XS +
+                                                                        (size_t)Ns * SSD_XS + 2 * SSD_L);
+  static size_t lds_allowed = 64 * 1024;
+  if (lds > lds_allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)ssd_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(160 * 1024));
+    if (e != hipSuccess) return (int)e;
+    lds_allowed = 160 * 1024;
+  }
+  const dim3 grid((unsigned)(nh * (P / SSD_PW)), (unsigned)B);
+  ssd_chunk_kernel<<<grid, 256, lds, stream>>>((const bf16_t*)xbc, xbc_stride, (const bf16_t*)dt_raw, dt_stride, dt_bias,
+                                               a_log, skip, state, state_stride, y, seq_starts, state_slots, nh, P, Ns, G, NP);
+  IA_LAUNCH_CHECK();
+  return IA_OK;
+}
+
 // ------------------------------------------------------------------------------------------ gate and norm
 // One workgroup per (row, part): out = unit_rms(y * silu(z)) * w over the part's `size` values.
 template <typename T>
@@ -444,6 +642,7 @@ IA_OP(ia_causal_conv)
 IA_OP(ia_conv_state_update)
 IA_OP(ia_qk_prepare)
 IA_OP(ia_ssd_scan)
+IA_OP(ia_ssd_chunked)
 IA_OP(ia_gated_group_norm)
 IA_OP(ia_concat_cast)
 IA_OP(ia_stream_add)

@@ -1048,6 +1048,38 @@ def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_l
     return y
 
 
+# tokens of portions in a step from which the recurrence runs as matrix products over chunks
+SSD_CHUNKED_FROM = 64
+
+
+def ssd_chunked_takes(dtype: torch.dtype, nh: int, P: int, Ns: int, G: int, xbc_stride: int) -> bool:
+    """Whether :func:`ssd_chunked` has a kernel for these sizes: bf16 rows, P a multiple of 16, a state of a multiple
+    of 16 up to 256."""
+    return dtype == torch.bfloat16 and bool(_core().ia_ssd_chunked_takes(int(nh), int(P), int(Ns), int(G), int(xbc_stride)))
+
+
+def ssd_chunked(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, skip: torch.Tensor,
+                state: torch.Tensor, y: torch.Tensor, seq_starts: torch.Tensor, state_slots: torch.Tensor, nh: int, P: int,
+                Ns: int, G: int) -> torch.Tensor:
+    """What :func:`ssd_scan` computes, as matrix products over chunks of 64 tokens of every request (fp32 but for the
+    product of C with B, whose bf16 operands are the stored values): for steps with portions of prompts.  The sums
+    are taken in another order than token after token, so results differ from :func:`ssd_scan` by fp32 rounding."""
+    N, B = xbc.shape[0], state_slots.numel()
+    _rows(xbc, nh * P + 2 * G * Ns, "ssd_chunked xbc")
+    _rows(dt_raw, nh, "ssd_chunked dt")
+    _need(dt_raw.dtype == xbc.dtype and dt_raw.shape[0] == N, "ssd_chunked: dt rows of xbc's dtype")
+    _need(ssd_chunked_takes(xbc.dtype, nh, P, Ns, G, xbc.stride(0)), "ssd_chunked: sizes that it does not take")
+    for t, what in ((dt_bias, "dt_bias"), (a_log, "a_log"), (skip, "skip")):
+        _f32(t, nh, "ssd_chunked " + what)
+    _need(y.is_cuda and y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (N, nh * P),
+          "ssd_chunked: y [N, nh P] fp32")
+    stride = _state_rows(state, nh * Ns * P, "ssd_chunked")
+    _ok(_core().ia_ssd_chunked(_p(xbc), DTYPE_CODE[xbc.dtype], xbc.stride(0), _p(dt_raw), dt_raw.stride(0), _p(dt_bias),
+                               _p(a_log), _p(skip), _p(state), ctypes.c_long(stride), _p(y), _p(seq_starts),
+                               _p(state_slots), B, nh, P, Ns, G, _stream()), "ssd_chunked")
+    return y
+
+
 def gated_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
                      out: torch.Tensor) -> torch.Tensor:
     """out = unit_rms(y * silu(z)) * w, the root mean square taken over each of ``groups`` equal parts of a row."""

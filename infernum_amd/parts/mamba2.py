@@ -75,6 +75,12 @@ class Mamba2Mixer(Mixer):
             raise K.KernelError("mamba2 needs a state slot")
         return cache.state, cache.state[:, self.conv_floats:]
 
+    def _chunked(self, xbc: torch.Tensor, portion_tokens: int) -> bool:
+        """Steps that bring enough tokens of prompts run the recurrence as matrix products over chunks (where
+        there is a kernel for the sizes); the others, decode steps among them, token after token from registers."""
+        return portion_tokens >= K.SSD_CHUNKED_FROM and K.ssd_chunked_takes(xbc.dtype, self.nh, self.P, self.Ns, self.G,
+                                                                           int(xbc.stride(0)))
+
     # ---- one step --------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: CacheView):
         n, dev, inner, cd = x.shape[0], x.device, self.inner, self.conv_dim
@@ -87,8 +93,9 @@ class Mamba2Mixer(Mixer):
         if self.taps > 1:
             K.conv_state_update(u, self.taps, conv_state, ctx.seq_starts, ctx.state_slots)
         y = torch.empty((n, inner), dtype=torch.float32, device=dev)
-        K.ssd_scan(xbc, proj[:, inner + cd:], self.dt_bias, self.a_log, self.skip, ssm_state, y, ctx.seq_starts,
-                   ctx.state_slots, self.nh, self.P, self.Ns, self.G)
+        scan = K.ssd_chunked if self._chunked(xbc, ctx.num_tokens - ctx.num_decode) else K.ssd_scan
+        scan(xbc, proj[:, inner + cd:], self.dt_bias, self.a_log, self.skip, ssm_state, y, ctx.seq_starts,
+             ctx.state_slots, self.nh, self.P, self.Ns, self.G)
         gated = torch.empty((n, inner), dtype=self.rt.dtype, device=dev)
         K.gated_group_norm(y, proj[:, :inner], self.w_norm, self.norm_groups, self.norm_eps, gated)
         return linear(gated, self.w_o, keep_split=True, kernels=self.rt.kernels)
@@ -96,7 +103,7 @@ class Mamba2Mixer(Mixer):
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not Mamba2Mixer.forward:
             return super().native(program, view)
-        from ..engine.program import STREAM
+        from ..engine.program import STREAM, Guard
         rt, inner, cd, row, taps = self.rt, self.inner, self.conv_dim, self.row, self.taps
         act, ab, N, T = program.act_code, program.act_bytes, program.N, program.T
         state, _ = self._states(view)
@@ -111,9 +118,14 @@ class Mamba2Mixer(Mixer):
             program.op("core", "ia_conv_state_update", [u, act, row, None, state, stride, program.seq_starts,
                                                         program.state_slots, program.B, cd, taps, STREAM])
         y = program.buffer("mamba2.y", T * inner * 4)
-        program.op("core", "ia_ssd_scan", [xbc, act, cd, dt, row, self.dt_bias, self.a_log, self.skip, ssm, stride, y,
-                                           program.seq_starts, program.state_slots, program.B, self.nh, self.P, self.Ns,
-                                           self.G, STREAM])
+        args = [xbc, act, cd, dt, row, self.dt_bias, self.a_log, self.skip, ssm, stride, y, program.seq_starts,
+                program.state_slots, program.B, self.nh, self.P, self.Ns, self.G, STREAM]
+        if K.ssd_chunked_takes(rt.dtype, self.nh, self.P, self.Ns, self.G, cd):
+            long = Guard.between(program.NPT, K.SSD_CHUNKED_FROM)
+            program.op("core", "ia_ssd_chunked", args, long)
+            program.op("core", "ia_ssd_scan", args, ~long)
+        else:
+            program.op("core", "ia_ssd_scan", args)
         gated = program.buffer("mamba2.gated", T * inner * ab)
         program.op("core", "ia_gated_group_norm", [y, proj, act, row, self.w_norm, gated, N, inner, self.norm_groups,
                                                    float(self.norm_eps), STREAM])

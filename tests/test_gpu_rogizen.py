@@ -133,6 +133,62 @@ def test_norm_and_rotation_of_queries_and_keys(dtype, nh, nkv, d, rot, pairing, 
         assert torch.equal(v_pages[page, :, :, off].float().cpu(), x[t, nh * d:].view(nkv, d))
 
 
+def _plain_recurrence(x, Bm, Cm, dt_raw, dt_bias, a_log, skip, S0):
+    """x [T, nh, P], Bm and Cm [T, G, N], dt_raw [T, nh], S0 [nh, N, P], all float64: (y [T, nh, P], S after T)."""
+    T, nh, P = x.shape
+    per = nh // Bm.shape[1]
+    dt = PR.softplus(dt_raw + dt_bias)
+    decay = torch.exp(-torch.exp(a_log)[None, :] * dt)
+    S, y = S0.clone(), torch.zeros(T, nh, P, dtype=torch.float64)
+    for t in range(T):
+        Bh, Ch = Bm[t].repeat_interleave(per, 0), Cm[t].repeat_interleave(per, 0)
+        S = decay[t][:, None, None] * S + dt[t][:, None, None] * Bh[:, :, None] * x[t][:, None, :]
+        y[t] = (S * Ch[:, :, None]).sum(1) + skip[:, None] * x[t]
+    return y, S
+
+
+@pytest.mark.parametrize("nh,P,Ns,G", [(4, 48, 32, 2), (2, 16, 16, 1), (3, 64, 128, 3), (8, 32, 80, 2), (1, 16, 256, 1)])
+@pytest.mark.parametrize("kernel", ["token_by_token", "chunks"])
+def test_recurrence_over_requests_of_unequal_length(nh, P, Ns, G, kernel):
+    """Requests of 1, 63, 64, 65, 130 and 200 tokens in one step, each from a state that is not zero, in slots out of
+    order: outputs and the states left behind, against the plain recurrence.  Both kernels: token after token, and
+    matrix products over chunks of 64 (a chunk's last row, the first of the next, a partial last chunk, a single
+    token).  One head forgets slowly, so that the state a chunk hands on carries weight."""
+    from infernum_amd.kernels import api as K
+    lens, slots = (1, 63, 64, 65, 130, 200), [4, 0, 6, 1, 3, 5]
+    T, cd = sum(lens), nh * P + 2 * G * Ns
+    g = torch.Generator().manual_seed(nh * 100 + Ns)
+    xbc = (torch.randn(T, cd, generator=g) * 0.7).to(torch.bfloat16)
+    dt_raw = torch.randn(T, nh + 3, generator=g).to(torch.bfloat16)[:, :nh]
+    dt_bias, a_log, skip = torch.rand(nh, generator=g) - 1.0, torch.rand(nh, generator=g) * 2 - 1.0, torch.rand(nh, generator=g) + 0.5
+    a_log[0] = -6.0
+    state0 = torch.randn(7, nh * Ns * P + 5, generator=g)
+    state = state0.to(DEV)[:, 2:2 + nh * Ns * P]
+    assert K.ssd_chunked_takes(torch.bfloat16, nh, P, Ns, G, cd)
+    seq, starts, sl = _ctx(lens, slots)
+    y = torch.full((T, nh * P), 7.0, device=DEV)
+    run = K.ssd_chunked if kernel == "chunks" else K.ssd_scan
+    run(xbc.to(DEV), dt_raw.to(DEV), dt_bias.to(DEV), a_log.to(DEV), skip.to(DEV), state, y, starts, sl, nh, P, Ns, G)
+    p = 0
+    for n, slot in zip(lens, slots):
+        rows = xbc[p:p + n].double()
+        want, S = _plain_recurrence(rows[:, :nh * P].view(n, nh, P), rows[:, nh * P:nh * P + G * Ns].view(n, G, Ns),
+                                    rows[:, nh * P + G * Ns:].view(n, G, Ns), dt_raw[p:p + n].double(), dt_bias.double(),
+                                    a_log.double(), skip.double(), state0[slot, 2:2 + nh * Ns * P].double().view(nh, Ns, P))
+        assert rel_err(y[p:p + n], want.view(n, -1)) <= 2e-5, (n, slot)
+        assert rel_err(state[slot], S.view(-1)) <= 2e-5, (n, slot)
+        p += n
+    assert torch.equal(state[2].cpu(), state0[2, 2:2 + nh * Ns * P])           # a slot of no request stays
+
+
+def test_sizes_the_chunked_recurrence_leaves_to_the_other_kernel():
+    from infernum_amd.kernels import api as K
+    assert not K.ssd_chunked_takes(torch.float32, 4, 48, 32, 2, 320)           # 32-bit steps go token after token
+    assert not K.ssd_chunked_takes(torch.bfloat16, 4, 10, 32, 2, 168)          # a head of 10 values
+    assert not K.ssd_chunked_takes(torch.bfloat16, 4, 16, 5, 4, 104)           # a state of 5
+    assert not K.ssd_chunked_takes(torch.bfloat16, 1, 16, 512, 1, 1040)        # a state past 256
+
+
 @BOTH
 @pytest.mark.parametrize("inner,parts,n", [(48, 3, 5), (40, 1, 70), (128, 2, 3), (96, 6, 33), (2048, 8, 4)])
 def test_gate_then_norm_in_parts(dtype, inner, parts, n):
