@@ -22,7 +22,7 @@
 #include "common.h"
 
 // ------------------------------------------------------------------------------------------ convolution
-// u [N, >= C] (stride u_stride), state [slots, taps-1, C] fp32: state[slot][j] is the input at position
+// w [C, taps], or [taps, C] with tap_major.  u [N, >= C] (stride u_stride), state [slots, taps-1, C] fp32: state[slot][j] is the input at position
 // ctx - (taps-1) + j of the request (zero before its start: a slot is cleared when it is taken).
 // y[t] = b_out + sum_j w[c, j] (u[t - (taps-1) + j] + b_in), j ascending.
 template <typename TU, typename TY>
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     const TU* __restrict__ u, int u_stride, const float* __restrict__ bias_in, const float* __restrict__ w,
     const float* __restrict__ bias_out, int act, TY* __restrict__ y, int y_stride, const float* __restrict__ state,
     long state_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_starts,
-    const int* __restrict__ state_slots, int N, int C, int taps) {
+    const int* __restrict__ state_slots, int N, int C, int taps, int tap_major) {
   const int r = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (r >= N || c >= C) return;
@@ -46,10 +46,64 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
       v = to_float(u[(size_t)(r - lag) * u_stride + c]) + b_in;
     else
       v = st[(size_t)(i - lag + taps - 1) * C + c];
-    acc = __builtin_fmaf(w[(size_t)c * taps + j], v, acc);
+    acc = __builtin_fmaf(tap_major ? w[(size_t)j * C + c] : w[(size_t)c * taps + j], v, acc);
   }
   if (act == 1) acc = acc / (1.f + expf(-acc));
   y[(size_t)r * y_stride + c] = from_float<TY>(acc);
+}
+
+// The same for bf16 rows whose channels come in whole 16-byte pieces and weights stored tap by tap ([taps, C]: the
+// weights of neighbouring channels are neighbours): a thread takes 8 channels of a row, the additions in the order
+// of causal_conv_kernel.
+__global__ __launch_bounds__(256) void causal_conv_vec_kernel(
+    const bf16_t* __restrict__ u, int u_stride, const float* __restrict__ bias_in, const float* __restrict__ w,
+    const float* __restrict__ bias_out, int act, bf16_t* __restrict__ y, int y_stride, const float* __restrict__ state,
+    long state_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_starts,
+    const int* __restrict__ state_slots, int N, int C, int taps) {
+  const int r = blockIdx.y;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (r >= N || c >= C) return;
+  const int s = token_seq[r];
+  const int i = r - seq_starts[s];
+  const float* st = state + (size_t)state_slots[s] * state_stride;
+  float b_in[8], acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    b_in[e] = bias_in ? bias_in[c + e] : 0.f;
+    acc[e] = bias_out ? bias_out[c + e] : 0.f;
+  }
+  for (int j = 0; j < taps; ++j) {
+    const int lag = taps - 1 - j;
+    float v[8];
+    if (i - lag >= 0) {
+      const uint4 p = *(const uint4*)(u + (size_t)(r - lag) * u_stride + c);
+      const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(pw[e] << 16) + b_in[2 * e];
+        v[2 * e + 1] = __uint_as_float(pw[e] & 0xffff0000u) + b_in[2 * e + 1];
+      }
+    } else {
+      const float* sp = st + (size_t)(i - lag + taps - 1) * C + c;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = sp[e];
+    }
+    const float4 w0 = *(const float4*)(w + (size_t)j * C + c), w1 = *(const float4*)(w + (size_t)j * C + c + 4);
+    const float wj[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wj[e], v[e], acc[e]);
+  }
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float a = acc[2 * e], b = acc[2 * e + 1];
+    if (act == 1) {
+      a = a / (1.f + expf(-a));
+      b = b / (1.f + expf(-b));
+    }
+    o[e] = (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+  }
+  *(uint4*)(y + (size_t)r * y_stride + c) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // After the step: state[slot][j] <- the input at position ctx + q - (taps-1) + j, from this step's rows or from the
@@ -78,15 +132,23 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
 extern "C" int ia_causal_conv(const void* u, int u_code, int u_stride, const float* bias_in, const float* w,
                               const float* bias_out, int act, void* y, int y_code, int y_stride, const float* state,
                               long state_stride, const int* token_seq, const int* seq_starts, const int* state_slots, int N, int C,
-                              int taps, hipStream_t stream) {
+                              int taps, int tap_major, hipStream_t stream) {
   if (N == 0) return IA_OK;
   if (!u || !w || !y || !state || !token_seq || !seq_starts || !state_slots || C <= 0 || taps < 1 || u_stride < C ||
       y_stride < C || N < 0 || N > 65535 || state_stride < (long)(taps - 1) * C || (act != 0 && act != 1))
     return IA_ERR_BAD_ARG;
+  if (tap_major && u_code == IA_BF16 && y_code == IA_BF16 && C % 8 == 0 && !((uintptr_t)w & 15) && u_stride % 8 == 0 && y_stride % 8 == 0 &&
+      !((uintptr_t)u & 15) && !((uintptr_t)y & 15)) {
+    const dim3 vgrid((unsigned)((C / 8 + 255) / 256), (unsigned)N);
+    causal_conv_vec_kernel<<<vgrid, 256, 0, stream>>>((const bf16_t*)u, u_stride, bias_in, w, bias_out, act, (bf16_t*)y,
+                                                      y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps);
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
   const dim3 grid((unsigned)((C + 255) / 256), (unsigned)N);
 #define IA_CONV(TU, TY)                                                                                          \
   causal_conv_kernel<TU, TY><<<grid, 256, 0, stream>>>((const TU*)u, u_stride, bias_in, w, bias_out, act, (TY*)y, \
-                                                       y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps)
+                                                       y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps, tap_major)
   if (u_code == IA_F32 && y_code == IA_F32) IA_CONV(float, float);
   else if (u_code == IA_BF16 && y_code == IA_BF16) IA_CONV(bf16_t, bf16_t);
   else if (u_code == IA_F32 && y_code == IA_BF16) IA_CONV(float, bf16_t);
@@ -336,6 +398,9 @@ typedef float sm_f32x4 __attribute__((ext_vector_type(4)));
 #define SSD_GS 68         // row stride of the chunk's [L, L] matrix in LDS, floats
 #define SSD_XS 20         // row stride of x and of the state in LDS, floats
 
+// What a thread holds of the next chunk while the current one is computed.
+#define SSD_MAXV 4        // 16-byte pieces of B (and of C) a thread loads per chunk: 64 rows of up to 128 values
+
 __global__ __launch_bounds__(256) void ssd_chunk_kernel(
     const bf16_t* __restrict__ xbc, int xbc_stride, const bf16_t* __restrict__ dt_raw, int dt_stride,
     const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ skip,
@@ -348,8 +413,10 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(
   float* Gs = (float*)(Cs + SSD_L * BS);                   // [L][GS]
   float* Xs = Gs + SSD_L * SSD_GS;                         // [L][XS]
   float* Ss = Xs + SSD_L * SSD_XS;                         // [Ns][XS]
-  float* cum = Ss + (size_t)Ns * SSD_XS;                   // [L]
-  float* dts = cum + SSD_L;                                // [L]
+  float* cum = Ss + (size_t)Ns * SSD_XS;                   // [L] running sum of a
+  float* dts = cum + SSD_L;                                // [L] step sizes
+  float* ecs = dts + SSD_L;                                // [L] exp(c_i)
+  float* wts = ecs + SSD_L;                                // [L] exp(c_L - c_j) dt_j
   const int slices = P / SSD_PW;
   const int hd = blockIdx.x / slices, ps = blockIdx.x - hd * slices;
   const int s = blockIdx.y;
@@ -372,30 +439,61 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(
       Bs[r * BS + c] = 0;
       Cs[r * BS + c] = 0;
     }
-  const int vec_row = Ns >> 3;                             // 16-byte pieces of a row of B or C
+  // a thread's pieces of a chunk: piece v of B and C is 8 values of row (tid + 256 v) / vec_row; x values 4 tid .. 4 tid + 3
+  const int vec_row = Ns >> 3;                             // 16-byte pieces of a row of B or C (a power of two or not)
+  int vr[SSD_MAXV], vc[SSD_MAXV];
+#pragma unroll
+  for (int v = 0; v < SSD_MAXV; ++v) {
+    const int i = tid + 256 * v;
+    vr[v] = i / vec_row;
+    vc[v] = 8 * (i - vr[v] * vec_row);
+    if (vr[v] >= SSD_L) vr[v] = -1;
+  }
+  const int xr = tid >> 2, xc = 4 * (tid & 3);
+  uint4 nb_[SSD_MAXV], nc_[SSD_MAXV];
+  uint2 nx_;
+  float ndt;
+  auto fetch = [&](int c0) {                               // the chunk's rows from memory into registers
+    const int Lc = q - c0 < SSD_L ? q - c0 : SSD_L;
+    const size_t row0 = (size_t)(first + c0);
+#pragma unroll
+    for (int v = 0; v < SSD_MAXV; ++v) {
+      nb_[v] = make_uint4(0, 0, 0, 0);
+      nc_[v] = nb_[v];
+      if (vr[v] >= 0 && vr[v] < Lc) {
+        const bf16_t* rp = xbc + (row0 + vr[v]) * xbc_stride;
+        nb_[v] = *(const uint4*)(rp + b_col + vc[v]);
+        nc_[v] = *(const uint4*)(rp + c_col + vc[v]);
+      }
+    }
+    nx_ = make_uint2(0, 0);
+    if (xr < Lc) nx_ = *(const uint2*)(xbc + (row0 + xr) * xbc_stride + x_col + xc);
+    ndt = 0.f;
+    if (wave == 0 && lane < Lc) ndt = to_float(dt_raw[(row0 + lane) * dt_stride + hd]);
+  };
+  fetch(0);
   for (int c0 = 0; c0 < q; c0 += SSD_L) {
     const int Lc = q - c0 < SSD_L ? q - c0 : SSD_L;
     const size_t row0 = (size_t)(first + c0);
     __syncthreads();                                       // the chunk before is done with B, C, x and the sums
-    // ---- B, C, x of the chunk; step sizes and the running sum of a
-    for (int i = tid; i < SSD_L * vec_row; i += 256) {
-      const int r = i / vec_row, v = i - r * vec_row;
-      uint4 bv = make_uint4(0, 0, 0, 0), cv = bv;
-      if (r < Lc) {
-        bv = *(const uint4*)(xbc + (row0 + r) * xbc_stride + b_col + 8 * v);
-        cv = *(const uint4*)(xbc + (row0 + r) * xbc_stride + c_col + 8 * v);
+    // ---- B, C, x of the chunk from the registers; step sizes, the running sum of a and what hangs on it
+#pragma unroll
+    for (int v = 0; v < SSD_MAXV; ++v)
+      if (vr[v] >= 0) {
+        *(uint4*)(Bs + vr[v] * BS + vc[v]) = nb_[v];
+        *(uint4*)(Cs + vr[v] * BS + vc[v]) = nc_[v];
       }
-      *(uint4*)(Bs + r * BS + 8 * v) = bv;
-      *(uint4*)(Cs + r * BS + 8 * v) = cv;
-    }
-    for (int i = tid; i < SSD_L * SSD_PW; i += 256) {
-      const int r = i >> 4, c = i & 15;
-      Xs[r * SSD_XS + c] = r < Lc ? to_float(xbc[(row0 + r) * xbc_stride + x_col + c]) : 0.f;
+    {
+      float* xp = Xs + xr * SSD_XS + xc;
+      xp[0] = __uint_as_float(nx_.x << 16);
+      xp[1] = __uint_as_float(nx_.x & 0xffff0000u);
+      xp[2] = __uint_as_float(nx_.y << 16);
+      xp[3] = __uint_as_float(nx_.y & 0xffff0000u);
     }
     if (wave == 0) {
       float dt = 0.f;
       if (lane < Lc) {
-        const float z = to_float(dt_raw[(row0 + lane) * dt_stride + hd]) + bias;
+        const float z = ndt + bias;
         dt = z > 20.f ? z : log1pf(expf(z));
       }
       float c = A * dt;
@@ -404,77 +502,108 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(
         const float up = __shfl_up(c, o, 64);
         if (lane >= o) c += up;
       }
+      const float clast = __shfl(c, 63, 64);
       cum[lane] = c;
       dts[lane] = dt;
+      ecs[lane] = expf(c);
+      wts[lane] = expf(clast - c) * dt;
     }
+    if (c0 + SSD_L < q) fetch(c0 + SSD_L);                 // the next chunk is on its way while this one is computed
     __syncthreads();
-    // ---- G[i][j] = (C_i . B_j) exp(c_i - c_j) dt_j for j <= i: wave w makes rows 16 w .. 16 w + 15
-    for (int jt = 0; jt <= wave; ++jt) {
-      sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      const uint16_t* cp = Cs + (16 * wave + l15) * BS + 8 * kk;
+    // ---- G[i][j] = (C_i . B_j) exp(c_i - c_j) dt_j for j <= i: the ten tiles of 16 x 16 on and under the diagonal,
+    // wave w takes tiles w, w + 4, w + 8 of the list (0,0) (1,0) (1,1) (2,0) ... (3,3)
+    for (int t = wave; t < 10; t += 4) {
+      const int it = t < 1 ? 0 : t < 3 ? 1 : t < 6 ? 2 : 3;
+      const int jt = t - (it * (it + 1) >> 1);
+      sm_f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+      const uint16_t* cp = Cs + (16 * it + l15) * BS + 8 * kk;
       const uint16_t* bp = Bs + (16 * jt + l15) * BS + 8 * kk;
-      for (int k0 = 0; k0 < NP; k0 += 32) {
-        const sm_bf16x8 a = *(const sm_bf16x8*)(cp + k0);
-        const sm_bf16x8 b = *(const sm_bf16x8*)(bp + k0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+      for (int k0 = 0; k0 < NP; k0 += 64) {
+        const sm_bf16x8 a0 = *(const sm_bf16x8*)(cp + k0), b0 = *(const sm_bf16x8*)(bp + k0);
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc0, 0, 0, 0);
+        if (k0 + 32 < NP) {
+          const sm_bf16x8 a1 = *(const sm_bf16x8*)(cp + k0 + 32), b1 = *(const sm_bf16x8*)(bp + k0 + 32);
+          acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc1, 0, 0, 0);
+        }
       }
       const int j = 16 * jt + l15;
       const float cj = cum[j], dj = dts[j];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int i = 16 * wave + 4 * kk + r;
-        Gs[i * SSD_GS + j] = j <= i ? acc[r] * expf(cum[i] - cj) * dj : 0.f;
+        const int i = 16 * it + 4 * kk + r;
+        Gs[i * SSD_GS + j] = j <= i ? (acc0[r] + acc1[r]) * expf(cum[i] - cj) * dj : 0.f;
       }
     }
     __syncthreads();
-    // ---- y rows 16 w .. 16 w + 15 of the chunk: G x + exp(c_i) C S0 + D x
+    // ---- y rows 16 w .. 16 w + 15 of the chunk: G x + exp(c_i) C S0 + D x, in three sums that run side by side
     {
-      sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      sm_f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc1 = acc, acc2 = acc;
       const int i = 16 * wave + l15;                       // the row this lane feeds
       for (int jb = 0; jb <= wave; ++jb) {
         const sm_f32x4 a = *(const sm_f32x4*)(Gs + i * SSD_GS + 16 * jb + 4 * kk);
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], Xs[(16 * jb + 4 * kk + r) * SSD_XS + l15], acc, 0, 0, 0);
+        const float* xp = Xs + (16 * jb + 4 * kk) * SSD_XS + l15;
+        const float x0 = xp[0], x1 = xp[SSD_XS], x2 = xp[2 * SSD_XS], x3 = xp[3 * SSD_XS];
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], x0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], x1, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], x2, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], x3, acc, 0, 0, 0);
       }
-      const float ei = expf(cum[i]);
-      for (int nb = 0; nb < Ns; nb += 16) {
+      const float ei = ecs[i];
+      for (int nb = 0; nb < Ns; nb += 32) {
+        const bool two = nb + 16 < Ns;
         const uint2 cw = *(const uint2*)(Cs + i * BS + nb + 4 * kk);
-        const float a0 = __uint_as_float(cw.x << 16) * ei, a1 = __uint_as_float(cw.x & 0xffff0000u) * ei;
-        const float a2 = __uint_as_float(cw.y << 16) * ei, a3 = __uint_as_float(cw.y & 0xffff0000u) * ei;
+        const uint2 cv = two ? *(const uint2*)(Cs + i * BS + nb + 16 + 4 * kk) : make_uint2(0, 0);
         const float* sp = Ss + (nb + 4 * kk) * SSD_XS + l15;
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, sp[0], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, sp[SSD_XS], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a2, sp[2 * SSD_XS], acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a3, sp[3 * SSD_XS], acc, 0, 0, 0);
+        const float* sq = two ? sp + 16 * SSD_XS : sp;
+        const float s0 = sp[0], s1 = sp[SSD_XS], s2 = sp[2 * SSD_XS], s3 = sp[3 * SSD_XS];
+        const float t0 = sq[0], t1 = sq[SSD_XS], t2 = sq[2 * SSD_XS], t3 = sq[3 * SSD_XS];
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cw.x << 16) * ei, s0, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cv.x << 16) * ei, t0, acc2, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cw.x & 0xffff0000u) * ei, s1, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cv.x & 0xffff0000u) * ei, t1, acc2, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cw.y << 16) * ei, s2, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cv.y << 16) * ei, t2, acc2, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cw.y & 0xffff0000u) * ei, s3, acc1, 0, 0, 0);
+        acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(cv.y & 0xffff0000u) * ei, t3, acc2, 0, 0, 0);
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int io = 16 * wave + 4 * kk + r;
         if (io < Lc)
-          y[(row0 + io) * yw + x_col + l15] = __builtin_fmaf(D, Xs[io * SSD_XS + l15], acc[r]);
+          y[(row0 + io) * yw + x_col + l15] = __builtin_fmaf(D, Xs[io * SSD_XS + l15], acc[r] + (acc1[r] + acc2[r]));
       }
     }
     __syncthreads();                                       // every wave has read S0
-    // ---- the state after the chunk: tiles of 16 state rows, wave w takes tiles w, w + 4, ...
+    // ---- the state after the chunk: tiles of 16 state rows, wave w takes tiles w, w + 4, ..., two at a time
     {
-      const float clast = cum[SSD_L - 1];
-      const float keep = expf(clast);
-      for (int nt = wave; 16 * nt < Ns; nt += 4) {
-        sm_f32x4 acc;
+      const float keep = ecs[SSD_L - 1];
+      for (int nt = wave; 16 * nt < Ns; nt += 8) {
+        const bool two = 16 * (nt + 4) < Ns;
+        const int nu = two ? nt + 4 : nt;
+        sm_f32x4 acc, acc1;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] = keep * Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15];
+        for (int r = 0; r < 4; ++r) {
+          acc[r] = keep * Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15];
+          acc1[r] = keep * Ss[(16 * nu + 4 * kk + r) * SSD_XS + l15];
+        }
+#pragma unroll 2
         for (int jb = 0; jb < SSD_L; jb += 16) {
+          const sm_f32x4 wj = *(const sm_f32x4*)(wts + jb + 4 * kk);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int j = jb + 4 * kk + r;
-            const float wj = expf(clast - cum[j]) * dts[j];
-            const float a = __uint_as_float((uint32_t)Bs[j * BS + 16 * nt + l15] << 16) * wj;
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Xs[j * SSD_XS + l15], acc, 0, 0, 0);
+            const float xv = Xs[j * SSD_XS + l15];
+            const float a = __uint_as_float((uint32_t)Bs[j * BS + 16 * nt + l15] << 16) * wj[r];
+            const float a1 = __uint_as_float((uint32_t)Bs[j * BS + 16 * nu + l15] << 16) * wj[r];
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a, xv, acc, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, xv, acc1, 0, 0, 0);
           }
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15] = acc[r];
+        for (int r = 0; r < 4; ++r) {
+          Ss[(16 * nt + 4 * kk + r) * SSD_XS + l15] = acc[r];
+          if (two) Ss[(16 * nu + 4 * kk + r) * SSD_XS + l15] = acc1[r];
+        }
       }
     }
   }
@@ -484,7 +613,7 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(
 
 // Whether ia_ssd_chunked takes these sizes (otherwise ia_ssd_scan does the step).
 extern "C" int ia_ssd_chunked_takes(int nh, int P, int Ns, int G, int xbc_stride) {
-  return nh > 0 && G > 0 && nh % G == 0 && P % SSD_PW == 0 && Ns % 16 == 0 && Ns >= 16 && Ns <= 256 && xbc_stride % 8 == 0;
+  return nh > 0 && G > 0 && nh % G == 0 && P % SSD_PW == 0 && Ns % 16 == 0 && Ns >= 16 && Ns <= 32 * SSD_MAXV && xbc_stride % 8 == 0;
 }
 
 extern "C" int ia_ssd_chunked(const void* xbc, int code, int xbc_stride, const void* dt_raw, int dt_stride,
@@ -499,7 +628,7 @@ extern "C" int ia_ssd_chunked(const void* xbc, int code, int xbc_stride, const v
   if (code != IA_BF16 || !ia_ssd_chunked_takes(nh, P, Ns, G, xbc_stride)) return IA_ERR_UNSUPPORTED;
   const int NP = (Ns + 31) / 32 * 32;
   const size_t lds = 2 * (size_t)SSD_L * (NP + 8) * 2 + sizeof(float) * ((size_t)SSD_L * SSD_GS + (size_t)SSD_L * SSD_XS +
-                                                                        (size_t)Ns * SSD_XS + 2 * SSD_L);
+                                                                        (size_t)Ns * SSD_XS + 4 * SSD_L);
   static size_t lds_allowed = 64 * 1024;
   if (lds > lds_allowed) {
     hipError_t e = hipFuncSetAttribute((const void*)ssd_chunk_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(160 * 1024));

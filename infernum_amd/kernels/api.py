@@ -956,12 +956,13 @@ def _state_rows(state: torch.Tensor, need: int, what: str) -> int:
 def causal_conv(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, ctx_token_seq: torch.Tensor,
                 seq_starts: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
                 bias_in: Optional[torch.Tensor] = None, bias_out: Optional[torch.Tensor] = None,
-                activation: Optional[str] = None) -> torch.Tensor:
+                activation: Optional[str] = None, tap_major: bool = False) -> torch.Tensor:
     """out[t, c] = act(bias_out[c] + sum_j w[c, j] (u[t - (taps-1) + j, c] + bias_in[c])) over each request's own
     tokens; the inputs before this step's rows come from ``state`` [slots, >= (taps-1) C] fp32 (the request's last
     taps-1 inputs, zero before its start).  ``u`` and ``out`` may be column ranges of wider rows.  The state is
-    left as it was: :func:`conv_state_update` moves it on."""
-    N, (C, taps) = u.shape[0], w.shape
+    left as it was: :func:`conv_state_update` moves it on.  ``tap_major``: ``w`` is stored [taps, C], which lets
+    bf16 rows of whole 16-byte pieces run eight channels a thread."""
+    N, (C, taps) = u.shape[0], (w.shape[::-1] if tap_major else w.shape)
     _rows(u, C, "causal_conv input")
     _rows(out, C, "causal_conv output")
     _need(out.shape[0] == N and u.shape[1] == C and out.shape[1] == C, "causal_conv: u and out are [N, C]")
@@ -973,7 +974,7 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, ctx_token
     _ok(_core().ia_causal_conv(_p(u), DTYPE_CODE[u.dtype], u.stride(0), _p(bias_in), _p(w), _p(bias_out),
                                CONV_ACTIVATIONS[activation], _p(out), DTYPE_CODE[out.dtype], out.stride(0), _p(state),
                                ctypes.c_long(stride), _p(ctx_token_seq), _p(seq_starts), _p(state_slots), N, C, taps,
-                               _stream()), "causal_conv")
+                               int(bool(tap_major)), _stream()), "causal_conv")
     return out
 
 
@@ -1054,7 +1055,7 @@ SSD_CHUNKED_FROM = 64
 
 def ssd_chunked_takes(dtype: torch.dtype, nh: int, P: int, Ns: int, G: int, xbc_stride: int) -> bool:
     """Whether :func:`ssd_chunked` has a kernel for these sizes: bf16 rows, P a multiple of 16, a state of a multiple
-    of 16 up to 256."""
+    of 16 up to 128."""
     return dtype == torch.bfloat16 and bool(_core().ia_ssd_chunked_takes(int(nh), int(P), int(Ns), int(G), int(xbc_stride)))
 
 

@@ -65,7 +65,7 @@ class ConvAttention(Attention):
         self.w_o = tensors["o"].contiguous()
         self.b_qk = torch.cat([f32("q.b"), f32("k.b")]).contiguous()
         self.b_o = f32("o.b")
-        self.w_conv = torch.cat([f32("q.conv"), f32("k.conv")], dim=0).contiguous()
+        self.w_conv = torch.cat([f32("q.conv"), f32("k.conv")], dim=0).t().contiguous()      # tap by tap: [taps, channels]
         self.q_norm = f32("q.norm") if self.qk_norm else None
         self.k_norm = f32("k.norm") if self.qk_norm else None
         prepare_weights(self.rt, [(self.w_qk, None, False), (self.w_o, None, False)])
@@ -86,7 +86,8 @@ class ConvAttention(Attention):
         state = self._state(cache)
         u = linear(x, self.w_qk, kernels=self.rt.kernels)
         y = torch.empty_like(u)
-        K.causal_conv(u, self.w_conv, state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, y, bias_in=self.b_qk)
+        K.causal_conv(u, self.w_conv, state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, y, bias_in=self.b_qk,
+                      tap_major=True)
         if self.taps > 1:
             K.conv_state_update(u, self.taps, state, ctx.seq_starts, ctx.state_slots, bias_in=self.b_qk)
         q = torch.empty((n, nh * d), dtype=self.rt.dtype, device=dev)
@@ -112,7 +113,7 @@ class ConvAttention(Attention):
         u = emit_linear(program, program.x, N, self.w_qk, rt.dtype, None, False, "conv_attention.u", "conv_attention.qk").tensor()
         y = program.buffer("conv_attention.y", T * C * program.act_bytes)
         program.op("core", "ia_causal_conv", [u, act, C, self.b_qk, self.w_conv, None, 0, y, act, C, state, stride,
-                                              program.token_seq, program.seq_starts, program.state_slots, N, C, taps, STREAM])
+                                              program.token_seq, program.seq_starts, program.state_slots, N, C, taps, 1, STREAM])
         if taps > 1:
             program.op("core", "ia_conv_state_update", [u, act, C, self.b_qk, state, stride, program.seq_starts,
                                                         program.state_slots, program.B, C, taps, STREAM])

@@ -64,7 +64,7 @@ class Mamba2Mixer(Mixer):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         f32 = lambda name: tensors[name].to(torch.float32).contiguous()            # noqa: E731
         self.w_in, self.w_o = tensors["in"].contiguous(), tensors["o"].contiguous()
-        self.w_conv, self.b_conv = f32("conv"), f32("conv.b")
+        self.w_conv, self.b_conv = f32("conv").t().contiguous(), f32("conv.b")        # tap by tap: [taps, channels]
         self.dt_bias, self.a_log, self.skip, self.w_norm = f32("dt_bias"), f32("A_log"), f32("D"), f32("norm")
         prepare_weights(self.rt, [(self.w_in, None, False), (self.w_o, None, True)])
 
@@ -89,7 +89,7 @@ class Mamba2Mixer(Mixer):
         u = proj[:, inner:inner + cd]
         xbc = torch.empty((n, cd), dtype=self.rt.dtype, device=dev)
         K.causal_conv(u, self.w_conv, conv_state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, xbc,
-                      bias_out=self.b_conv, activation="silu")
+                      bias_out=self.b_conv, activation="silu", tap_major=True)
         if self.taps > 1:
             K.conv_state_update(u, self.taps, conv_state, ctx.seq_starts, ctx.state_slots)
         y = torch.empty((n, inner), dtype=torch.float32, device=dev)
@@ -113,7 +113,7 @@ class Mamba2Mixer(Mixer):
         proj = emit_linear(program, program.x, N, self.w_in, rt.dtype, None, False, "mamba2.proj", "mamba2.in").tensor()
         u, dt, xbc = proj.at(inner * ab), proj.at((inner + cd) * ab), program.buffer("mamba2.xbc", T * cd * ab)
         program.op("core", "ia_causal_conv", [u, act, row, None, self.w_conv, self.b_conv, 1, xbc, act, cd, state, stride,
-                                              program.token_seq, program.seq_starts, program.state_slots, N, cd, taps, STREAM])
+                                              program.token_seq, program.seq_starts, program.state_slots, N, cd, taps, 1, STREAM])
         if taps > 1:
             program.op("core", "ia_conv_state_update", [u, act, row, None, state, stride, program.seq_starts,
                                                         program.state_slots, program.B, cd, taps, STREAM])

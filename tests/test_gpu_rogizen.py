@@ -55,11 +55,14 @@ def _ctx(lengths, slots=None):
 
 # ------------------------------------------------------------------------------------ kernels alone
 @BOTH
-@pytest.mark.parametrize("C,taps", [(5, 1), (70, 2), (300, 4), (64, 7)])
-def test_convolution_with_its_state(dtype, C, taps):
+@pytest.mark.parametrize("C,taps", [(5, 1), (70, 2), (300, 4), (64, 7), (2056, 4)])
+@pytest.mark.parametrize("tap_major", [False, True])
+def test_convolution_with_its_state(dtype, C, taps, tap_major):
     """Three requests of unequal length beside each other, fed in two steps: the second step's first rows read the
     first step's last taps-1 inputs from the slots (slots not in the order of the requests), a request shorter than
-    the taps reads zeros and its own rows; biases on both sides; the input a column range of wider rows."""
+    the taps reads zeros and its own rows; biases on both sides; the input a column range of wider rows (at a
+    16-byte border when the channels come in eights: the kernel of eight channels a thread); weights stored channel
+    by channel or tap by tap."""
     from infernum_amd.kernels import api as K
     rt = runtime(dtype)
     lens1, lens2 = (1, 9, 2), (3, 1, 6)
@@ -72,13 +75,13 @@ def test_convolution_with_its_state(dtype, C, taps):
     got = [[], [], []]
     for step, lens in enumerate((lens1, lens2)):
         rows = torch.cat([u[(0 if step == 0 else lens1[i]):(lens1[i] if step == 0 else None)] for i, u in enumerate(us)])
-        wide = torch.full((rows.shape[0], C + 9), 7.0)
-        wide[:, 4:4 + C] = rows
-        u_dev = wide.to(DEV).to(rt.dtype)[:, 4:4 + C]
+        wide = torch.full((rows.shape[0], C + 16), 7.0)
+        wide[:, 8:8 + C] = rows
+        u_dev = wide.to(DEV).to(rt.dtype)[:, 8:8 + C]
         seq, starts, sl = _ctx(lens, slots)
         out = torch.empty((rows.shape[0], C), dtype=rt.dtype, device=DEV)
-        K.causal_conv(u_dev, w.to(DEV), state, seq, starts, sl, out, bias_in=b_in.to(DEV), bias_out=b_out.to(DEV),
-                      activation="silu")
+        K.causal_conv(u_dev, (w.t().contiguous() if tap_major else w).to(DEV), state, seq, starts, sl, out,
+                      bias_in=b_in.to(DEV), bias_out=b_out.to(DEV), activation="silu", tap_major=tap_major)
         if taps > 1:
             K.conv_state_update(u_dev, taps, state, starts, sl, bias_in=b_in.to(DEV))
         p = 0
@@ -147,7 +150,7 @@ def _plain_recurrence(x, Bm, Cm, dt_raw, dt_bias, a_log, skip, S0):
     return y, S
 
 
-@pytest.mark.parametrize("nh,P,Ns,G", [(4, 48, 32, 2), (2, 16, 16, 1), (3, 64, 128, 3), (8, 32, 80, 2), (1, 16, 256, 1)])
+@pytest.mark.parametrize("nh,P,Ns,G", [(4, 48, 32, 2), (2, 16, 16, 1), (3, 64, 128, 3), (8, 32, 80, 2), (1, 16, 112, 1)])
 @pytest.mark.parametrize("kernel", ["token_by_token", "chunks"])
 def test_recurrence_over_requests_of_unequal_length(nh, P, Ns, G, kernel):
     """Requests of 1, 63, 64, 65, 130 and 200 tokens in one step, each from a state that is not zero, in slots out of
@@ -186,7 +189,7 @@ def test_sizes_the_chunked_recurrence_leaves_to_the_other_kernel():
     assert not K.ssd_chunked_takes(torch.float32, 4, 48, 32, 2, 320)           # 32-bit steps go token after token
     assert not K.ssd_chunked_takes(torch.bfloat16, 4, 10, 32, 2, 168)          # a head of 10 values
     assert not K.ssd_chunked_takes(torch.bfloat16, 4, 16, 5, 4, 104)           # a state of 5
-    assert not K.ssd_chunked_takes(torch.bfloat16, 1, 16, 512, 1, 1040)        # a state past 256
+    assert not K.ssd_chunked_takes(torch.bfloat16, 1, 16, 256, 1, 528)         # a state past 128
 
 
 @BOTH
