@@ -66,11 +66,14 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(
   const int s = token_seq[r];
   const int i = r - seq_starts[s];
   const float* st = state + (size_t)state_slots[s] * state_stride;
-  float b_in[8], acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    b_in[e] = bias_in ? bias_in[c + e] : 0.f;
-    acc[e] = bias_out ? bias_out[c + e] : 0.f;
+  float b_in[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (bias_in) {
+    const float4 lo = *(const float4*)(bias_in + c), hi = *(const float4*)(bias_in + c + 4);
+    b_in[0] = lo.x, b_in[1] = lo.y, b_in[2] = lo.z, b_in[3] = lo.w, b_in[4] = hi.x, b_in[5] = hi.y, b_in[6] = hi.z, b_in[7] = hi.w;
+  }
+  if (bias_out) {
+    const float4 lo = *(const float4*)(bias_out + c), hi = *(const float4*)(bias_out + c + 4);
+    acc[0] = lo.x, acc[1] = lo.y, acc[2] = lo.z, acc[3] = lo.w, acc[4] = hi.x, acc[5] = hi.y, acc[6] = hi.z, acc[7] = hi.w;
   }
   for (int j = 0; j < taps; ++j) {
     const int lag = taps - 1 - j;
@@ -137,7 +140,8 @@ extern "C" int ia_causal_conv(const void* u, int u_code, int u_stride, const flo
   if (!u || !w || !y || !state || !token_seq || !seq_starts || !state_slots || C <= 0 || taps < 1 || u_stride < C ||
       y_stride < C || N < 0 || N > 65535 || state_stride < (long)(taps - 1) * C || (act != 0 && act != 1))
     return IA_ERR_BAD_ARG;
-  if (tap_major && u_code == IA_BF16 && y_code == IA_BF16 && C % 8 == 0 && !((uintptr_t)w & 15) && u_stride % 8 == 0 && y_stride % 8 == 0 &&
+  if (tap_major && u_code == IA_BF16 && y_code == IA_BF16 && C % 8 == 0 && !((uintptr_t)w & 15) &&
+      !((uintptr_t)bias_in & 15) && !((uintptr_t)bias_out & 15) && u_stride % 8 == 0 && y_stride % 8 == 0 &&
       !((uintptr_t)u & 15) && !((uintptr_t)y & 15)) {
     const dim3 vgrid((unsigned)((C / 8 + 255) / 256), (unsigned)N);
     causal_conv_vec_kernel<<<vgrid, 256, 0, stream>>>((const bf16_t*)u, u_stride, bias_in, w, bias_out, act, (bf16_t*)y,
@@ -666,12 +670,52 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __re
   }
 }
 
+// The same for parts of up to 256 PER values: a thread keeps its gated values between the sum and the store (one
+// pass over y and z); the additions in the order of gated_group_norm_kernel.
+template <typename T, int PER>
+__global__ __launch_bounds__(256) void gated_group_norm_kept_kernel(const float* __restrict__ y, const T* __restrict__ z,
+                                                                    int z_stride, const float* __restrict__ w,
+                                                                    T* __restrict__ out, int inner, int size, float eps) {
+  __shared__ float red[4];
+  const int r = blockIdx.y, part = blockIdx.x;
+  const size_t base = (size_t)part * size;
+  float v[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    v[k] = 0.f;
+    if (i < size) {
+      const float g = to_float(z[(size_t)r * z_stride + base + i]);
+      v[k] = y[(size_t)r * inner + base + i] * (g / (1.f + expf(-g)));
+      ss = __builtin_fmaf(v[k], v[k], ss);
+    }
+  }
+  ss = block_sum<256>(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + 256 * k;
+    if (i < size) out[(size_t)r * inner + base + i] = from_float<T>(v[k] * inv * w[base + i]);
+  }
+}
+
 extern "C" int ia_gated_group_norm(const float* y, const void* z, int code, int z_stride, const float* w, void* out,
                                    int N, int inner, int groups, float eps, hipStream_t stream) {
   if (N == 0) return IA_OK;
   if (!y || !z || !w || !out || N < 0 || N > 65535 || inner <= 0 || groups <= 0 || inner % groups || z_stride < inner)
     return IA_ERR_BAD_ARG;
   const dim3 grid((unsigned)groups, (unsigned)N);
+  const int size = inner / groups;
+  if (size <= 1024 && (code == IA_F32 || code == IA_BF16)) {
+#define IA_GGN(T, PER)                                                                                                  \
+  gated_group_norm_kept_kernel<T, PER><<<grid, 256, 0, stream>>>(y, (const T*)z, z_stride, w, (T*)out, inner, size, eps)
+    if (code == IA_F32) { if (size <= 256) IA_GGN(float, 1); else if (size <= 512) IA_GGN(float, 2); else IA_GGN(float, 4); }
+    else { if (size <= 256) IA_GGN(bf16_t, 1); else if (size <= 512) IA_GGN(bf16_t, 2); else IA_GGN(bf16_t, 4); }
+#undef IA_GGN
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
   if (code == IA_F32)
     gated_group_norm_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)z, z_stride, w, (float*)out, inner,
                                                             inner / groups, eps);

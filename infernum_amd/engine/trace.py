@@ -33,7 +33,7 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, stream: IO
           file=sys.stderr, flush=True)
     engine = Engine.from_pretrained(
         model_dir, dtype=dtype,
-        cache_config=CacheConfig(page_size=page_size, num_pages=num_pages, num_state_slots=2 * MAX_LIVE_REQUESTS,
+        cache_config=CacheConfig(page_size=page_size, num_pages=num_pages, num_state_slots=MAX_LIVE_REQUESTS,
                                  poison_freed_pages=poison),
         max_tokens_per_step=max(8192, int(max_tokens)), kernels=kernels)
     print(f"[trace_run] ready: {num_pages} pages of {page_size} tokens", file=sys.stderr, flush=True)
