@@ -109,6 +109,93 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(
   *(uint4*)(y + (size_t)r * y_stride + c) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
+// The same again for steps of many rows and at most four taps: a thread takes 8 channels of CONV_ROWS consecutive
+// rows, loads every input row once for all the rows that reach it, and the weights once.
+#define CONV_ROWS 4
+__global__ __launch_bounds__(256) void causal_conv_rows_kernel(
+    const bf16_t* __restrict__ u, int u_stride, const float* __restrict__ bias_in, const float* __restrict__ w,
+    const float* __restrict__ bias_out, int act, bf16_t* __restrict__ y, int y_stride, const float* __restrict__ state,
+    long state_stride, const int* __restrict__ token_seq, const int* __restrict__ seq_starts,
+    const int* __restrict__ state_slots, int N, int C, int taps) {
+  const int r0 = blockIdx.y * CONV_ROWS;
+  const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (r0 >= N || c >= C) return;
+  float b_in[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, b_out[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (bias_in) {
+    const float4 lo = *(const float4*)(bias_in + c), hi = *(const float4*)(bias_in + c + 4);
+    b_in[0] = lo.x, b_in[1] = lo.y, b_in[2] = lo.z, b_in[3] = lo.w, b_in[4] = hi.x, b_in[5] = hi.y, b_in[6] = hi.z, b_in[7] = hi.w;
+  }
+  if (bias_out) {
+    const float4 lo = *(const float4*)(bias_out + c), hi = *(const float4*)(bias_out + c + 4);
+    b_out[0] = lo.x, b_out[1] = lo.y, b_out[2] = lo.z, b_out[3] = lo.w, b_out[4] = hi.x, b_out[5] = hi.y, b_out[6] = hi.z, b_out[7] = hi.w;
+  }
+  // input rows r0 - 3 .. r0 + CONV_ROWS - 1 of the step (those that exist), with the input bias
+  float in[CONV_ROWS + 3][8];
+#pragma unroll
+  for (int k = 0; k < CONV_ROWS + 3; ++k) {
+    const int r = r0 - 3 + k;
+    uint4 p = make_uint4(0, 0, 0, 0);
+    if (r >= 0 && r < N) p = *(const uint4*)(u + (size_t)r * u_stride + c);
+    const uint32_t pw[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      in[k][2 * e] = __uint_as_float(pw[e] << 16) + b_in[2 * e];
+      in[k][2 * e + 1] = __uint_as_float(pw[e] & 0xffff0000u) + b_in[2 * e + 1];
+    }
+  }
+  // the weights by how far back their tap reaches (lag 0: the row itself), so that every index is known to the compiler
+  float wt[4][8];
+#pragma unroll
+  for (int lag = 0; lag < 4; ++lag) {
+    float4 w0 = make_float4(0.f, 0.f, 0.f, 0.f), w1 = w0;
+    if (lag < taps) {
+      w0 = *(const float4*)(w + (size_t)(taps - 1 - lag) * C + c);
+      w1 = *(const float4*)(w + (size_t)(taps - 1 - lag) * C + c + 4);
+    }
+    wt[lag][0] = w0.x, wt[lag][1] = w0.y, wt[lag][2] = w0.z, wt[lag][3] = w0.w;
+    wt[lag][4] = w1.x, wt[lag][5] = w1.y, wt[lag][6] = w1.z, wt[lag][7] = w1.w;
+  }
+#pragma unroll
+  for (int k = 0; k < CONV_ROWS; ++k) {
+    const int r = r0 + k;
+    if (r < N) {
+      const int s = token_seq[r];
+      const int i = r - seq_starts[s];
+      const float* st = state + (size_t)state_slots[s] * state_stride;
+      float acc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = b_out[e];
+#pragma unroll
+      for (int lag = 3; lag >= 0; --lag) {               // taps in ascending order
+        if (lag < taps) {
+          float v[8];
+          if (i - lag >= 0) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = in[k + 3 - lag][e];
+          } else {
+            const float* sp = st + (size_t)(i - lag + taps - 1) * C + c;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = sp[e];
+          }
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wt[lag][e], v[e], acc[e]);
+        }
+      }
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float a = acc[2 * e], b = acc[2 * e + 1];
+        if (act == 1) {
+          a = a / (1.f + expf(-a));
+          b = b / (1.f + expf(-b));
+        }
+        o[e] = (uint32_t)float_to_bf16_bits(a) | ((uint32_t)float_to_bf16_bits(b) << 16);
+      }
+      *(uint4*)(y + (size_t)r * y_stride + c) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 // After the step: state[slot][j] <- the input at position ctx + q - (taps-1) + j, from this step's rows or from the
 // old state (read in ascending j before the places are written: a thread owns its channel's taps-1 values).
 template <typename TU>
@@ -143,6 +230,13 @@ extern "C" int ia_causal_conv(const void* u, int u_code, int u_stride, const flo
   if (tap_major && u_code == IA_BF16 && y_code == IA_BF16 && C % 8 == 0 && !((uintptr_t)w & 15) &&
       !((uintptr_t)bias_in & 15) && !((uintptr_t)bias_out & 15) && u_stride % 8 == 0 && y_stride % 8 == 0 &&
       !((uintptr_t)u & 15) && !((uintptr_t)y & 15)) {
+    if (taps <= 4 && N >= 64) {
+      const dim3 rgrid((unsigned)((C / 8 + 255) / 256), (unsigned)((N + CONV_ROWS - 1) / CONV_ROWS));
+      causal_conv_rows_kernel<<<rgrid, 256, 0, stream>>>((const bf16_t*)u, u_stride, bias_in, w, bias_out, act, (bf16_t*)y,
+                                                         y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps);
+      IA_LAUNCH_CHECK();
+      return IA_OK;
+    }
     const dim3 vgrid((unsigned)((C / 8 + 255) / 256), (unsigned)N);
     causal_conv_vec_kernel<<<vgrid, 256, 0, stream>>>((const bf16_t*)u, u_stride, bias_in, w, bias_out, act, (bf16_t*)y,
                                                       y_stride, state, state_stride, token_seq, seq_starts, state_slots, N, C, taps);

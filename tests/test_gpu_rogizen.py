@@ -57,15 +57,15 @@ def _ctx(lengths, slots=None):
 @BOTH
 @pytest.mark.parametrize("C,taps", [(5, 1), (70, 2), (300, 4), (64, 7), (2056, 4)])
 @pytest.mark.parametrize("tap_major", [False, True])
-def test_convolution_with_its_state(dtype, C, taps, tap_major):
+@pytest.mark.parametrize("lens1,lens2", [((1, 9, 2), (3, 1, 6)), ((40, 30, 2), (3, 70, 65))])
+def test_convolution_with_its_state(dtype, C, taps, tap_major, lens1, lens2):
     """Three requests of unequal length beside each other, fed in two steps: the second step's first rows read the
     first step's last taps-1 inputs from the slots (slots not in the order of the requests), a request shorter than
     the taps reads zeros and its own rows; biases on both sides; the input a column range of wider rows (at a
-    16-byte border when the channels come in eights: the kernel of eight channels a thread); weights stored channel
-    by channel or tap by tap."""
+    16-byte border when the channels come in eights: the kernel of eight channels a thread, and from 64 rows on
+    the one that takes four rows a thread); weights stored channel by channel or tap by tap."""
     from infernum_amd.kernels import api as K
     rt = runtime(dtype)
-    lens1, lens2 = (1, 9, 2), (3, 1, 6)
     g = torch.Generator().manual_seed(C + taps)
     w, b_in, b_out = torch.randn(C, taps, generator=g), torch.randn(C, generator=g), torch.randn(C, generator=g)
     us = [_x(a + b, C, dtype, 20 + i) for i, (a, b) in enumerate(zip(lens1, lens2))]
