@@ -17,11 +17,12 @@ pytestmark = pytest.mark.gpu
 BOTH = pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 # largest |difference| of a logit as a fraction of the RMS of the plain logits (see test_gpu_engine.py)
 TOL = {"float32": 2e-5, "bfloat16": 6e-2}
-LENGTHS = {"R1": (1, 7, 45, 83, 130), "R2": (3, 61, 33, 97), "R3": (9, 70, 121), "R4": (2, 17, 38, 64, 150)}
+LENGTHS = {"R1": (1, 7, 45, 83, 130), "R2": (3, 61, 33, 97), "R3": (9, 70, 121), "R4": (2, 17, 38, 64, 150),
+           "R5": (1, 64, 65, 200), "R6": (5, 63, 129)}
 MIXED = {"R1": (70, 131, 64, 150, 33, 97, 66, 81), "R2": (150, 165, 120, 190, 147), "R3": (129, 65, 90, 47, 72, 99),
-         "R4": (70, 131, 64, 150, 33, 97, 66, 81)}
-PAGE = {"R1": 16, "R2": 4, "R3": 8, "R4": 16}
-NAMES = ["R1", "R2", "R3", "R4"]
+         "R4": (70, 131, 64, 150, 33, 97, 66, 81), "R5": (150, 100, 64, 190, 129, 77), "R6": (70, 131, 64, 150, 33, 97)}
+PAGE = {"R1": 16, "R2": 4, "R3": 8, "R4": 16, "R5": 16, "R6": 8}
+NAMES = ["R1", "R2", "R3", "R4", "R5", "R6"]
 # tolerance per configuration: three times what rounding alone costs the plain model (computed in 32-bit; for
 # bfloat16 with every stored activation rounded to bfloat16 besides), and at least TOL's.  The recurrent layers'
 # norm over a few values that nearly cancel, and states carried over a hundred tokens, make some places sensitive.
