@@ -4,6 +4,7 @@
 //                          request kept in its state slot (fp32), an optional bias on the input (a projection's),
 //                          an optional bias on the output and an optional silu
 //   ia_conv_state_update   the state of that convolution after a step
+//   ia_causal_conv_single  both at once for steps in which every request brings one token
 //   ia_qk_prepare          query and key heads between projection and attention: an RMS norm per head (one weight
 //                          for all heads), rotation of neighbouring or half-split pairs with a factor on sine and
 //                          cosine, the keys to their pages, and as values either the value heads of the row or the
@@ -217,6 +218,56 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
       v = st[(size_t)(j + q) * C + c];
     st[(size_t)j * C + c] = v;
   }
+}
+
+// For steps in which every request brings one token: the convolution and the state's move in one pass.  A thread
+// owns a channel of a request: it reads the taps-1 kept inputs, adds in the order of causal_conv_kernel, and writes
+// them back one place down with the new input last.
+template <typename TU, typename TY>
+__global__ __launch_bounds__(256) void causal_conv_single_kernel(
+    const TU* __restrict__ u, int u_stride, const float* __restrict__ bias_in, const float* __restrict__ w,
+    const float* __restrict__ bias_out, int act, TY* __restrict__ y, int y_stride, float* __restrict__ state,
+    long state_stride, const int* __restrict__ token_seq, const int* __restrict__ state_slots, int N, int C, int taps,
+    int tap_major) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (r >= N || c >= C) return;
+  float* st = state + (size_t)state_slots[token_seq[r]] * state_stride;
+  float acc = bias_out ? bias_out[c] : 0.f;
+  const float cur = to_float(u[(size_t)r * u_stride + c]) + (bias_in ? bias_in[c] : 0.f);
+  for (int j = 0; j < taps - 1; ++j) {
+    const float v = st[(size_t)j * C + c];
+    acc = __builtin_fmaf(tap_major ? w[(size_t)j * C + c] : w[(size_t)c * taps + j], v, acc);
+    if (j > 0) st[(size_t)(j - 1) * C + c] = v;
+  }
+  acc = __builtin_fmaf(tap_major ? w[(size_t)(taps - 1) * C + c] : w[(size_t)c * taps + taps - 1], cur, acc);
+  if (taps > 1) st[(size_t)(taps - 2) * C + c] = cur;
+  if (act == 1) acc = acc / (1.f + expf(-acc));
+  y[(size_t)r * y_stride + c] = from_float<TY>(acc);
+}
+
+// Every request of the step brings exactly one token (row r is request token_seq[r]'s): what ia_causal_conv and
+// ia_conv_state_update do one after the other, the same bits.
+extern "C" int ia_causal_conv_single(const void* u, int u_code, int u_stride, const float* bias_in, const float* w,
+                                     const float* bias_out, int act, void* y, int y_code, int y_stride, float* state,
+                                     long state_stride, const int* token_seq, const int* state_slots, int N, int C, int taps,
+                                     int tap_major, hipStream_t stream) {
+  if (N == 0) return IA_OK;
+  if (!u || !w || !y || !state || !token_seq || !state_slots || C <= 0 || taps < 1 || u_stride < C || y_stride < C ||
+      N < 0 || N > 65535 || state_stride < (long)(taps - 1) * C || (act != 0 && act != 1))
+    return IA_ERR_BAD_ARG;
+  const dim3 grid((unsigned)((C + 255) / 256), (unsigned)N);
+#define IA_CONV1(TU, TY)                                                                                               \
+  causal_conv_single_kernel<TU, TY><<<grid, 256, 0, stream>>>((const TU*)u, u_stride, bias_in, w, bias_out, act, (TY*)y, \
+                                                              y_stride, state, state_stride, token_seq, state_slots, N, C, taps, tap_major)
+  if (u_code == IA_F32 && y_code == IA_F32) IA_CONV1(float, float);
+  else if (u_code == IA_BF16 && y_code == IA_BF16) IA_CONV1(bf16_t, bf16_t);
+  else if (u_code == IA_F32 && y_code == IA_BF16) IA_CONV1(float, bf16_t);
+  else if (u_code == IA_BF16 && y_code == IA_F32) IA_CONV1(bf16_t, float);
+  else return IA_ERR_BAD_ARG;
+#undef IA_CONV1
+  IA_LAUNCH_CHECK();
+  return IA_OK;
 }
 
 extern "C" int ia_causal_conv(const void* u, int u_code, int u_stride, const float* bias_in, const float* w,
@@ -906,6 +957,7 @@ extern "C" int ia_softcap(float* x, int rows, int cols, float cap, hipStream_t s
 
 #include "op_call.h"
 IA_OP(ia_causal_conv)
+IA_OP(ia_causal_conv_single)
 IA_OP(ia_conv_state_update)
 IA_OP(ia_qk_prepare)
 IA_OP(ia_ssd_scan)

@@ -978,6 +978,29 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, ctx_token
     return out
 
 
+def causal_conv_single(u: torch.Tensor, w: torch.Tensor, state: torch.Tensor, ctx_token_seq: torch.Tensor,
+                       state_slots: torch.Tensor, out: torch.Tensor, bias_in: Optional[torch.Tensor] = None,
+                       bias_out: Optional[torch.Tensor] = None, activation: Optional[str] = None,
+                       tap_major: bool = False) -> torch.Tensor:
+    """:func:`causal_conv` and :func:`conv_state_update` in one pass for a step in which every request brings exactly
+    one token (row r belongs to request ``ctx_token_seq[r]``): the same bits, and the state is left moved on."""
+    N, (C, taps) = u.shape[0], (w.shape[::-1] if tap_major else w.shape)
+    _rows(u, C, "causal_conv_single input")
+    _rows(out, C, "causal_conv_single output")
+    _need(out.shape[0] == N and u.shape[1] == C and out.shape[1] == C, "causal_conv_single: u and out are [N, C]")
+    _f32(w, C * taps, "causal_conv_single weight")
+    _f32(bias_in, C, "causal_conv_single input bias")
+    _f32(bias_out, C, "causal_conv_single output bias")
+    stride = _state_rows(state, (taps - 1) * C, "causal_conv_single")
+    _i32(ctx_token_seq, N, "causal_conv_single token_seq")
+    _need(state_slots.numel() >= N, "causal_conv_single: a slot for every row's request")
+    _ok(_core().ia_causal_conv_single(_p(u), DTYPE_CODE[u.dtype], u.stride(0), _p(bias_in), _p(w), _p(bias_out),
+                                      CONV_ACTIVATIONS[activation], _p(out), DTYPE_CODE[out.dtype], out.stride(0),
+                                      _p(state), ctypes.c_long(stride), _p(ctx_token_seq), _p(state_slots), N, C, taps,
+                                      int(bool(tap_major)), _stream()), "causal_conv_single")
+    return out
+
+
 def conv_state_update(u: torch.Tensor, taps: int, state: torch.Tensor, seq_starts: torch.Tensor,
                       state_slots: torch.Tensor, bias_in: Optional[torch.Tensor] = None) -> None:
     """After :func:`causal_conv`: every request's state becomes its last taps-1 inputs, this step's included."""

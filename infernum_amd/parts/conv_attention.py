@@ -86,10 +86,13 @@ class ConvAttention(Attention):
         state = self._state(cache)
         u = linear(x, self.w_qk, kernels=self.rt.kernels)
         y = torch.empty_like(u)
-        K.causal_conv(u, self.w_conv, state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, y, bias_in=self.b_qk,
-                      tap_major=True)
-        if self.taps > 1:
-            K.conv_state_update(u, self.taps, state, ctx.seq_starts, ctx.state_slots, bias_in=self.b_qk)
+        if self.taps > 1 and ctx.num_decode == ctx.num_seqs:            # every request brings one token
+            K.causal_conv_single(u, self.w_conv, state, ctx.token_seq, ctx.state_slots, y, bias_in=self.b_qk, tap_major=True)
+        else:
+            K.causal_conv(u, self.w_conv, state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, y, bias_in=self.b_qk,
+                          tap_major=True)
+            if self.taps > 1:
+                K.conv_state_update(u, self.taps, state, ctx.seq_starts, ctx.state_slots, bias_in=self.b_qk)
         q = torch.empty((n, nh * d), dtype=self.rt.dtype, device=dev)
         K.qk_prepare(y, q, nh, nkv, d, ctx.positions, self.q_norm, self.k_norm, self.norm_eps, pos.inv_freq,
                      pos.rotary_dim if pos.inv_freq is not None else 0, pos.pairing, pos.magnitude, ctx.slots[g],
@@ -101,7 +104,7 @@ class ConvAttention(Attention):
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not ConvAttention.forward:
             return super(Attention, self).native(program, view)
-        from ..engine.program import ALWAYS, STREAM
+        from ..engine.program import ALWAYS, STREAM, Guard
         if view is None or view.k_pages is None or not view.writable:
             raise K.KernelError("conv_attention needs pages of its own")
         nh, nkv, d, rt, pos, C, taps = self.nh, self.nkv, self.d, self.rt, self.position, self.channels, self.taps
@@ -112,11 +115,16 @@ class ConvAttention(Attention):
         program.keep(self.w_qk, self.w_o, self.b_qk, self.b_o, self.w_conv, self.q_norm, self.k_norm, state, pos.inv_freq)
         u = emit_linear(program, program.x, N, self.w_qk, rt.dtype, None, False, "conv_attention.u", "conv_attention.qk").tensor()
         y = program.buffer("conv_attention.y", T * C * program.act_bytes)
+        portions = Guard.between(program.NP, 1) if taps > 1 else ALWAYS
         program.op("core", "ia_causal_conv", [u, act, C, self.b_qk, self.w_conv, None, 0, y, act, C, state, stride,
-                                              program.token_seq, program.seq_starts, program.state_slots, N, C, taps, 1, STREAM])
+                                              program.token_seq, program.seq_starts, program.state_slots, N, C, taps, 1,
+                                              STREAM], portions)
         if taps > 1:
             program.op("core", "ia_conv_state_update", [u, act, C, self.b_qk, state, stride, program.seq_starts,
-                                                        program.state_slots, program.B, C, taps, STREAM])
+                                                        program.state_slots, program.B, C, taps, STREAM], portions)
+            program.op("core", "ia_causal_conv_single", [u, act, C, self.b_qk, self.w_conv, None, 0, y, act, C, state, stride,
+                                                         program.token_seq, program.state_slots, N, C, taps, 1, STREAM],
+                       ~portions)
         q = program.buffer("attention.q", T * nh * d * program.act_bytes)
         rot = pos.rotary_dim if pos.inv_freq is not None else 0
         program.op("core", "ia_qk_prepare",

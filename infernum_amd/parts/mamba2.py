@@ -88,10 +88,14 @@ class Mamba2Mixer(Mixer):
         proj = linear(x, self.w_in, kernels=self.rt.kernels)                     # [n, z | x B C | dt]
         u = proj[:, inner:inner + cd]
         xbc = torch.empty((n, cd), dtype=self.rt.dtype, device=dev)
-        K.causal_conv(u, self.w_conv, conv_state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, xbc,
-                      bias_out=self.b_conv, activation="silu", tap_major=True)
-        if self.taps > 1:
-            K.conv_state_update(u, self.taps, conv_state, ctx.seq_starts, ctx.state_slots)
+        if self.taps > 1 and ctx.num_decode == ctx.num_seqs:            # every request brings one token
+            K.causal_conv_single(u, self.w_conv, conv_state, ctx.token_seq, ctx.state_slots, xbc, bias_out=self.b_conv,
+                                 activation="silu", tap_major=True)
+        else:
+            K.causal_conv(u, self.w_conv, conv_state, ctx.token_seq, ctx.seq_starts, ctx.state_slots, xbc,
+                          bias_out=self.b_conv, activation="silu", tap_major=True)
+            if self.taps > 1:
+                K.conv_state_update(u, self.taps, conv_state, ctx.seq_starts, ctx.state_slots)
         y = torch.empty((n, inner), dtype=torch.float32, device=dev)
         scan = K.ssd_chunked if self._chunked(xbc, ctx.num_tokens - ctx.num_decode) else K.ssd_scan
         scan(xbc, proj[:, inner + cd:], self.dt_bias, self.a_log, self.skip, ssm_state, y, ctx.seq_starts,
@@ -103,7 +107,7 @@ class Mamba2Mixer(Mixer):
     def native(self, program, view: CacheView) -> None:
         if type(self).forward is not Mamba2Mixer.forward:
             return super().native(program, view)
-        from ..engine.program import STREAM, Guard
+        from ..engine.program import ALWAYS, STREAM, Guard
         rt, inner, cd, row, taps = self.rt, self.inner, self.conv_dim, self.row, self.taps
         act, ab, N, T = program.act_code, program.act_bytes, program.N, program.T
         state, _ = self._states(view)
@@ -112,11 +116,16 @@ class Mamba2Mixer(Mixer):
         program.keep(state, ssm, self.w_conv, self.b_conv, self.dt_bias, self.a_log, self.skip, self.w_norm)
         proj = emit_linear(program, program.x, N, self.w_in, rt.dtype, None, False, "mamba2.proj", "mamba2.in").tensor()
         u, dt, xbc = proj.at(inner * ab), proj.at((inner + cd) * ab), program.buffer("mamba2.xbc", T * cd * ab)
+        portions = Guard.between(program.NP, 1) if taps > 1 else ALWAYS
         program.op("core", "ia_causal_conv", [u, act, row, None, self.w_conv, self.b_conv, 1, xbc, act, cd, state, stride,
-                                              program.token_seq, program.seq_starts, program.state_slots, N, cd, taps, 1, STREAM])
+                                              program.token_seq, program.seq_starts, program.state_slots, N, cd, taps, 1,
+                                              STREAM], portions)
         if taps > 1:
             program.op("core", "ia_conv_state_update", [u, act, row, None, state, stride, program.seq_starts,
-                                                        program.state_slots, program.B, cd, taps, STREAM])
+                                                        program.state_slots, program.B, cd, taps, STREAM], portions)
+            program.op("core", "ia_causal_conv_single", [u, act, row, None, self.w_conv, self.b_conv, 1, xbc, act, cd, state,
+                                                         stride, program.token_seq, program.state_slots, N, cd, taps, 1,
+                                                         STREAM], ~portions)
         y = program.buffer("mamba2.y", T * inner * 4)
         args = [xbc, act, cd, dt, row, self.dt_bias, self.a_log, self.skip, ssm, stride, y, program.seq_starts,
                 program.state_slots, program.B, self.nh, self.P, self.Ns, self.G, STREAM]

@@ -69,22 +69,33 @@ def test_convolution_with_its_state(dtype, C, taps, tap_major, lens1, lens2):
     rt = runtime(dtype)
     g = torch.Generator().manual_seed(C + taps)
     w, b_in, b_out = torch.randn(C, taps, generator=g), torch.randn(C, generator=g), torch.randn(C, generator=g)
-    us = [_x(a + b, C, dtype, 20 + i) for i, (a, b) in enumerate(zip(lens1, lens2))]
+    lens3 = (1, 1, 1)                       # a last step of single tokens: the kernel that moves the state as it goes
+    us = [_x(a + b + 1, C, dtype, 20 + i) for i, (a, b) in enumerate(zip(lens1, lens2))]
     want = [PR.silu(PR.causal_conv(u.double() + b_in.double(), w.double(), b_out.double())) for u in us]
     state = torch.zeros(8, max((taps - 1) * C, 1) + 3, device=DEV)[:, :max((taps - 1) * C, 1)]
     slots = [5, 0, 2]
     got = [[], [], []]
-    for step, lens in enumerate((lens1, lens2)):
-        rows = torch.cat([u[(0 if step == 0 else lens1[i]):(lens1[i] if step == 0 else None)] for i, u in enumerate(us)])
+    w_dev = (w.t().contiguous() if tap_major else w).to(DEV)
+    done = [0, 0, 0]
+    for step, lens in enumerate((lens1, lens2, lens3)):
+        rows = torch.cat([u[done[i]:done[i] + lens[i]] for i, u in enumerate(us)])
+        done = [d + n for d, n in zip(done, lens)]
         wide = torch.full((rows.shape[0], C + 16), 7.0)
         wide[:, 8:8 + C] = rows
         u_dev = wide.to(DEV).to(rt.dtype)[:, 8:8 + C]
         seq, starts, sl = _ctx(lens, slots)
         out = torch.empty((rows.shape[0], C), dtype=rt.dtype, device=DEV)
-        K.causal_conv(u_dev, (w.t().contiguous() if tap_major else w).to(DEV), state, seq, starts, sl, out,
-                      bias_in=b_in.to(DEV), bias_out=b_out.to(DEV), activation="silu", tap_major=tap_major)
-        if taps > 1:
-            K.conv_state_update(u_dev, taps, state, starts, sl, bias_in=b_in.to(DEV))
+        kw = dict(bias_in=b_in.to(DEV), bias_out=b_out.to(DEV), activation="silu", tap_major=tap_major)
+        if step == 2 and taps > 1:
+            twin, out2 = state.clone(), torch.empty_like(out)
+            K.causal_conv(u_dev, w_dev, twin, seq, starts, sl, out2, **kw)
+            K.conv_state_update(u_dev, taps, twin, starts, sl, bias_in=b_in.to(DEV))
+            K.causal_conv_single(u_dev, w_dev, state, seq, sl, out, **kw)
+            assert torch.equal(out, out2) and torch.equal(state, twin)          # the same bits both ways
+        else:
+            K.causal_conv(u_dev, w_dev, state, seq, starts, sl, out, **kw)
+            if taps > 1:
+                K.conv_state_update(u_dev, taps, state, starts, sl, bias_in=b_in.to(DEV))
         p = 0
         for i, n in enumerate(lens):
             got[i].append(out[p:p + n].float().cpu())
