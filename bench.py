@@ -499,13 +499,13 @@ def rogizen_configs(size: dict):
     attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
                  "conv": size["taps"], "scale": size["dim"] ** -0.5, "mask": {"size": size["chunk"]},
                  "rot": {"base": 10000.0, "dims": size["dim"] // 2,
-                         "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+                         "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     ssm = {"heads": size["ssm_heads"], "vdim": size["ssm_vdim"], "state": size["state"], "groups": size["groups"],
            "norm_groups": size["norm_groups"], "conv": size["taps"]}
     mlp = {"kind": "dense", "ff": size["ff"]}
     rog = RogizenConfig.from_dict({
         "architecture": "Rogizen", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
-        "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": {"start": 0, "stop": size["layers"], "times": 1},
+        "norm": {"eps": 1e-6}, "logit_softcap": 50.0, "loop": {"start": 0, "stop": size["layers"], "times": 1},
         "layers": [{"type": "attention", "mixer": attention, "mlp": mlp} if i % 4 == 3 else
                    {"type": "mamba2", "mixer": ssm, "mlp": mlp} for i in range(size["layers"])]})
     llama = LlamaConfig.from_dict(dict(

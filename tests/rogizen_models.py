@@ -11,9 +11,9 @@ R3: a loop of one layer that runs twice, entered at layer 0; twenty heads over o
     page; a convolution of one tap (nothing carried); a recurrent layer with a state of 64 x 64 a head.
 R4: the loop is the whole model and runs once; chunks of 37; no rotation at all; chunks of 1 (a query sees itself
     alone); five taps.
-R5: recurrent layers only (no pages at all), the second twice; heads of 48 values and a state of 32 (the chunked
-    recurrence's sizes); no feed-forward anywhere.
-R6: attention layers only, one tap (no state slot at all), the first three times; no mask in one, chunks of 64 in
+R5: recurrent layers only (no pages at all), the second twice; heads of 32 and 16 values and states of 48 and 16
+    (sizes the chunked recurrence takes); no feed-forward anywhere.
+R6: attention layers only, one tap (no state slot at all), the first three times; no mask in one, chunks of 32 in
     the other; a vocabulary larger than the width by far.
 """
 import json
@@ -56,7 +56,7 @@ R2 = {"architecture": "Rogizen", "vocab": 333, "width": 100, "embedding": {"scal
           _layer("mamba2", _ssm(4, 10, 5, 4, 1, 2)),
       ]}
 R3 = {"architecture": "Rogizen", "vocab": 256, "width": 128, "embedding": {"scale": 11.3}, "norm": {"eps": 3e-6},
-      "logit_softcap": 30.0, "loop": {"start": 0, "stop": 1, "times": 2},
+      "logit_softcap": 25.0, "loop": {"start": 0, "stop": 1, "times": 2},
       "layers": [
           _layer("mamba2", _ssm(2, 64, 64, 2, 1, 4), ff=200),
           _layer("attention", _attn(20, 1, 32, 1, chunk=16, rot={"base": 1000000.0, "dims": 16, "scaling": {
@@ -72,15 +72,15 @@ R4 = {"architecture": "Rogizen", "vocab": 300, "width": 96, "embedding": {"scale
 R5 = {"architecture": "Rogizen", "vocab": 150, "width": 80, "embedding": {"scale": 8.9}, "norm": {"eps": 1e-6},
       "logit_softcap": 20.0, "loop": {"start": 1, "stop": 2, "times": 2},
       "layers": [
-          _layer("mamba2", _ssm(2, 48, 32, 1, 2, 3)),
-          _layer("mamba2", _ssm(4, 48, 32, 2, 1, 4)),
+          _layer("mamba2", _ssm(2, 32, 48, 1, 2, 3)),
+          _layer("mamba2", _ssm(4, 16, 16, 2, 1, 4)),
       ]}
 R6 = {"architecture": "Rogizen", "vocab": 1100, "width": 48, "embedding": {"scale": 6.9}, "norm": {"eps": 1e-5},
       "logit_softcap": 15.0, "loop": {"start": 0, "stop": 1, "times": 3},
       "layers": [
           _layer("attention", _attn(3, 3, 16, 1, rot={"base": 500.0, "dims": 4}), ff=64),
-          _layer("attention", _attn(4, 2, 32, 1, chunk=64, rot={"base": 50000.0, "dims": 16, "scaling": {
-              "factor": 8.0, "original": 128, "fast": 16.0, "slow": 1.0}}, scale=0.2), None),
+          _layer("attention", _attn(4, 2, 32, 1, chunk=32, rot={"base": 40000.0, "dims": 8, "scaling": {
+              "factor": 6.0, "original": 128, "fast": 16.0, "slow": 1.5}}, scale=0.2), None),
       ]}
 RAW = {"R1": R1, "R2": R2, "R3": R3, "R4": R4, "R5": R5, "R6": R6}
 SEED = {"R1": 5, "R2": 6, "R3": 7, "R4": 15, "R5": 9, "R6": 10}

@@ -162,7 +162,7 @@ def _plain_recurrence(x, Bm, Cm, dt_raw, dt_bias, a_log, skip, S0):
     return y, S
 
 
-@pytest.mark.parametrize("nh,P,Ns,G", [(4, 48, 32, 2), (2, 16, 16, 1), (3, 64, 128, 3), (8, 32, 80, 2), (1, 16, 112, 1)])
+@pytest.mark.parametrize("nh,P,Ns,G", [(4, 32, 48, 2), (2, 16, 16, 1), (3, 64, 128, 3), (8, 32, 80, 2), (1, 16, 112, 1)])
 @pytest.mark.parametrize("kernel", ["token_by_token", "chunks"])
 def test_recurrence_over_requests_of_unequal_length(nh, P, Ns, G, kernel):
     """Requests of 1, 63, 64, 65, 130 and 200 tokens in one step, each from a state that is not zero, in slots out of
@@ -198,7 +198,7 @@ def test_recurrence_over_requests_of_unequal_length(nh, P, Ns, G, kernel):
 
 def test_sizes_the_chunked_recurrence_leaves_to_the_other_kernel():
     from infernum_amd.kernels import api as K
-    assert not K.ssd_chunked_takes(torch.float32, 4, 48, 32, 2, 320)           # 32-bit steps go token after token
+    assert not K.ssd_chunked_takes(torch.float32, 2, 32, 16, 1, 96)           # 32-bit steps go token after token
     assert not K.ssd_chunked_takes(torch.bfloat16, 4, 10, 32, 2, 168)          # a head of 10 values
     assert not K.ssd_chunked_takes(torch.bfloat16, 4, 16, 5, 4, 104)           # a state of 5
     assert not K.ssd_chunked_takes(torch.bfloat16, 1, 16, 256, 1, 528)         # a state past 128
