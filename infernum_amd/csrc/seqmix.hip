@@ -390,6 +390,82 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
 }
 
+// The same for bf16 heads of whole 16-byte pieces whose rotated pairs are neighbours (or that are not rotated):
+// a group of GL lanes (a power of two, at least d / 8) per (token, head), a lane takes 8 consecutive values, so a
+// pair lies within a lane and every access but the transposed values' is 16 bytes.
+__global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
+    const bf16_t* __restrict__ x, int x_stride, bf16_t* __restrict__ q_out, int q_stride, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float eps, const int* __restrict__ positions, const int* __restrict__ slots,
+    const void* __restrict__ freq, int freq_f64, int rot, float magnitude, bf16_t* __restrict__ k_pages,
+    bf16_t* __restrict__ v_pages, int N, int nh, int nkv, int d, int page_size, int num_pages, int values_are_keys, int GL) {
+  const int heads = nh + nkv;
+  const int per_block = 256 / GL;
+  const long item = (long)blockIdx.x * per_block + threadIdx.x / GL;
+  const int ch = threadIdx.x % GL;                        // which 8 values of the head
+  const bool in_range = item < (long)N * heads;           // lanes past the end go along for the shuffles, idle
+  const int t = in_range ? (int)(item / heads) : 0, hd = in_range ? (int)(item % heads) : 0;
+  const bool live = in_range && 8 * ch < d;
+  const bool is_key = hd >= nh;
+  const bf16_t* src = x + (size_t)t * x_stride + (size_t)hd * d + 8 * ch;
+  const float* wn = is_key ? k_norm : q_norm;
+  uint4 raw = make_uint4(0, 0, 0, 0);
+  if (live) raw = *(const uint4*)src;
+  const uint32_t rw[4] = {raw.x, raw.y, raw.z, raw.w};
+  float v[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[2 * e] = __uint_as_float(rw[e] << 16);
+    v[2 * e + 1] = __uint_as_float(rw[e] & 0xffff0000u);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ss = __builtin_fmaf(v[e], v[e], ss);
+  for (int o = GL >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, IA_WAVE);
+  if (!live || (is_key && !k_pages)) return;
+  const int slot = is_key ? slots[t] : 0;
+  const int page = slot / page_size, off = slot - page * page_size;
+  if (is_key && (page < 0 || page >= num_pages)) return;
+  const int g = hd - nh;
+  if (is_key) {
+    // the values: the value head of the row, or the key head as it came in; transposed within the page
+    uint4 vr = raw;
+    if (!values_are_keys) vr = *(const uint4*)(x + (size_t)t * x_stride + (size_t)(heads + g) * d + 8 * ch);
+    const uint32_t vw[4] = {vr.x, vr.y, vr.z, vr.w};
+    uint16_t* vdst = (uint16_t*)v_pages + ((size_t)page * nkv + g) * (size_t)d * page_size + (size_t)(8 * ch) * page_size + off;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      vdst[(size_t)(2 * e) * page_size] = (uint16_t)(vw[e] & 0xffffu);
+      vdst[(size_t)(2 * e + 1) * page_size] = (uint16_t)(vw[e] >> 16);
+    }
+  }
+  if (wn) {
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    const float4 w0 = *(const float4*)(wn + 8 * ch), w1 = *(const float4*)(wn + 8 * ch + 4);
+    const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * wv[e];
+  }
+  const int pos = positions[t];
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    if (8 * ch + e < rot) {
+      float sn, cs, lo, hi;
+      rope_sincos(pos, freq, freq_f64, (8 * ch + e) >> 1, sn, cs);
+      sn *= magnitude;
+      cs *= magnitude;
+      rope_pair(v[e], v[e + 1], cs, sn, lo, hi);
+      v[e] = lo;
+      v[e + 1] = hi;
+    }
+  }
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) o[e] = (uint32_t)float_to_bf16_bits(v[2 * e]) | ((uint32_t)float_to_bf16_bits(v[2 * e + 1]) << 16);
+  bf16_t* dst = is_key ? k_pages + (((size_t)page * nkv + g) * page_size + off) * d + 8 * ch
+                       : q_out + (size_t)t * q_stride + (size_t)hd * d + 8 * ch;
+  *(uint4*)dst = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 extern "C" int ia_qk_prepare(const void* x, int code, int x_stride, void* q_out, int q_stride, const float* q_norm,
                              const float* k_norm, float eps, const int* positions, const int* slots, const void* freq,
                              int freq_f64, int rot, int pairing, float magnitude, void* k_pages, void* v_pages, int N,
@@ -405,6 +481,18 @@ extern "C" int ia_qk_prepare(const void* x, int code, int x_stride, void* q_out,
   // the rotation reads its pair from the source and writes both places: in place only where source and
   // destination are the same element for element (q_out == x with equal strides), which this launch allows
   const long items = (long)N * (nh + nkv);
+  if (code == IA_BF16 && (pairing == 1 || rot == 0) && d % 8 == 0 && d <= 512 && x_stride % 8 == 0 && q_stride % 8 == 0 &&
+      !((uintptr_t)x & 15) && !((uintptr_t)q_out & 15) && !((uintptr_t)k_pages & 15) && !((uintptr_t)q_norm & 15) &&
+      !((uintptr_t)k_norm & 15)) {
+    int GL = 1;
+    while (8 * GL < d) GL <<= 1;
+    const int per_block = 256 / GL;
+    qk_prepare_vec_kernel<<<(unsigned)((items + per_block - 1) / per_block), 256, 0, stream>>>(
+        (const bf16_t*)x, x_stride, (bf16_t*)q_out, q_stride, q_norm, k_norm, eps, positions, slots, freq, freq_f64, rot,
+        magnitude, (bf16_t*)k_pages, (bf16_t*)v_pages, N, nh, nkv, d, page_size, num_pages, values_are_keys, GL);
+    IA_LAUNCH_CHECK();
+    return IA_OK;
+  }
   const unsigned grid = (unsigned)((items + 3) / 4);
   if (code == IA_F32)
     qk_prepare_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (float*)q_out, q_stride, q_norm, k_norm,

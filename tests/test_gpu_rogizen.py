@@ -107,7 +107,9 @@ def test_convolution_with_its_state(dtype, C, taps, tap_major, lens1, lens2):
 @BOTH
 @pytest.mark.parametrize("nh,nkv,d,rot,pairing,scaled", [(4, 2, 16, 8, "neighbours", True), (5, 5, 26, 26, "neighbours", False),
                                                          (3, 1, 32, 0, "neighbours", False), (2, 1, 80, 16, "half", False),
-                                                         (20, 1, 32, 16, "neighbours", True)])
+                                                         (20, 1, 32, 16, "neighbours", True), (16, 4, 128, 64, "neighbours", True),
+                                                         (3, 3, 48, 48, "neighbours", False), (2, 2, 64, 0, "neighbours", False),
+                                                         (1, 1, 256, 6, "neighbours", False)])
 def test_norm_and_rotation_of_queries_and_keys(dtype, nh, nkv, d, rot, pairing, scaled):
     """Queries against the plain norm and rotation at positions up to some thousands; keys in their pages, and the
     values there are the keys as they came in."""
